@@ -1,6 +1,7 @@
 """Reusable sublayers built on :mod:`fasttalk_llm_microservice_amd.ops.mixers`:
-latent attention (paged latent cache), windowed attention with sigmoid weights and
-windowed differential attention (paged key / value caches), the channel-decay gated
+latent attention (paged latent cache), windowed attention with sigmoid weights,
+windowed differential attention and convolved capped attention with a sink (paged key /
+value caches), the channel-decay gated
 delta rule and the selective state-space mixer (state slots), dense, gated and
 mixture-of-experts feed-forwards and the per-layer token-side input.
 
@@ -266,6 +267,46 @@ class DifferentialAttention(WindowedAttention):
         return F.linear(o, self.wo)
 
 
+class ConvSinkAttention(WindowedAttention):
+    """Grouped-query softmax attention over every earlier key (or a window of them) whose
+    q, k and v each pass a short per-channel causal convolution over time right after
+    their projection (no bias, no activation; the last taps-1 projected rows of a sequence
+    live in its state slot).  Each head's q and k are divided by their root mean square
+    and multiplied by one weight vector shared by all heads.  Positions do not enter the
+    scores: s = softcap tanh(q.k scale / softcap), and the softmax's denominator carries
+    one extra unit, exp(sink) with sink = 0 -- a key that is always visible and has no
+    value, so a row's weights may sum to less than one."""
+
+    def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
+                 scale: float, softcap: float, eps: float, dtype, device, window: int = 0,
+                 sink: Optional[float] = 0.0):
+        f32 = lambda n: get(n).to(device, torch.float32).contiguous()   # noqa: E731
+        spec = M.WindowSpec(heads, kv_heads, dim, vdim, int(window), float(scale), maps=1,
+                            softcap=float(softcap or 0.0), sink=sink)
+        wqkv = torch.cat([get("q"), get("k"), get("v")], 0).to(device, dtype).contiguous()
+        super().__init__(spec, wqkv, None, get("o").to(device, dtype).contiguous(), eps, dtype)
+        self.taps = int(taps)
+        self.conv_w = torch.cat([f32("q.conv"), f32("k.conv"), f32("v.conv")], 0).contiguous()
+        self.q_norm, self.k_norm = f32("q.norm"), f32("k.norm")
+        self.channels = self.nq + self.nk + self.nv
+        if wqkv.shape != (self.channels, width) or self.conv_w.shape != (self.channels, self.taps) \
+                or self.q_norm.numel() != dim or self.k_norm.numel() != dim:
+            raise ValueError("attention projections, convolutions or norms do not fit the head sizes")
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        """(paged keys, paged values, projected-row history per state slot)."""
+        return super().alloc_cache(num_blocks, block_size, dtype, num_slots, device) + \
+            _state_slots(((max(self.taps - 1, 0), self.channels),), num_slots, device)
+
+    def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
+        kc, vc, hist = cache
+        qkv = F.linear(h, self.wqkv)
+        q = M.conv_attn_prep(qkv, self.nq, self.nk, self.conv_w, hist, ctx.seg, self.q_norm, self.k_norm,
+                             self.eps, self.spec.dk, ctx.slot_mapping, kc, vc)
+        o = self.attend(q, ctx, (kc, vc))
+        return F.linear(o.view(h.shape[0], -1).to(self.dtype), self.wo)
+
+
 class StateSpaceMixer:
     """Selective state-space mixer with a scalar decay per head (state-space duality
     form): one input projection [z | x | B | C | dt], a short causal convolution with
@@ -340,37 +381,71 @@ def _glu_weights(get: Get, prefix: str, dtype, device, extra: Optional[torch.Ten
 
 
 class MoEFF:
-    """Top-k mixture of clamped-GLU experts with group-limited routing, an additive
-    selection bias that does not enter the weights, and an optional gated shared expert.
+    """Top-k mixture of small feed-forward experts with an optional shared expert that
+    runs for every token and is scaled by sigmoid(w_sg . h), one number per token.
 
-    Expert: g = min(W_gate h, limit), u = clamp(W_up h, +-limit),
-    y = g sigmoid(1.702 g) (u + 1), out = W_down y.  Router logits are fp32."""
+    Two designs of routing and expert are served (``routing`` / ``act``):
+
+    * ``"grouped_softmax"`` + ``"clamp_glu"``: softmax over all experts, an additive
+      selection bias (``correction``) that does not enter the weights, only the ``keep``
+      best of ``groups`` groups eligible; expert g = min(W_gate h, limit),
+      u = clamp(W_up h, +-limit), y = g sigmoid(1.702 g) (u + 1), out = W_down y;
+    * ``"top_logits"`` + ``"relu_sq"``: logits z = W_router h + b; the ``top`` largest are
+      chosen and weighted by the softmax over just those; expert out =
+      W_down relu(W_up h)^2.
+
+    Router logits are fp32 in both."""
 
     def __init__(self, get: Get, experts: int, top: int, limit: float, groups: int, keep: int,
-                 shared_limit: Optional[float], dtype, device):
+                 shared_limit: Optional[float], dtype, device, routing: str = "grouped_softmax",
+                 act: str = "clamp_glu", shared: Optional[bool] = None):
         if groups < 1 or experts % groups or not 1 <= keep <= groups or top > experts // groups * keep:
             raise ValueError("expert groups do not fit the expert count")
+        if routing not in ("grouped_softmax", "top_logits") or act not in ("clamp_glu", "relu_sq"):
+            raise ValueError("unknown routing or expert activation")
         self.e, self.top, self.limit, self.groups, self.keep = experts, top, float(limit), groups, keep
-        self.dtype = dtype
+        self.dtype, self.routing, self.act = dtype, routing, act
         self.router = get("router").to(device, torch.float32).contiguous()
-        self.correction = get("correction").to(device, torch.float32).contiguous()
-        gus, downs = zip(*[_glu_weights(get, f"e{i}.", dtype, device) for i in range(experts)])
-        self.wgu = torch.stack(gus).contiguous()       # [E, 2 ff, width]
-        self.wdown = torch.stack(downs).contiguous()   # [E, width, ff]
+        if routing == "grouped_softmax":
+            self.correction = get("correction").to(device, torch.float32).contiguous()
+            self.router_bias = None
+        else:
+            self.router_bias = get("router.b").to(device, torch.float32).contiguous()
+        if act == "clamp_glu":
+            firsts, downs = zip(*[_glu_weights(get, f"e{i}.", dtype, device) for i in range(experts)])
+        else:
+            firsts = [get(f"e{i}.up").to(device, dtype) for i in range(experts)]
+            downs = [get(f"e{i}.down").to(device, dtype) for i in range(experts)]
+        self.wgu = torch.stack(list(firsts)).contiguous()      # [E, 2 ff | ff, width]
+        self.wdown = torch.stack(list(downs)).contiguous()    # [E, width, ff]
         self.shared = None
-        if shared_limit is not None:
+        if shared is None:
+            shared = shared_limit is not None
+        if shared:
             # the shared expert's per-token gate logit rides as one more output row
-            self.shared = _glu_weights(get, "shared.", dtype, device, extra=get("shared.sg"))
-            self.shared_limit = float(shared_limit)
+            if act == "clamp_glu":
+                self.shared = _glu_weights(get, "shared.", dtype, device, extra=get("shared.sg"))
+            else:
+                self.shared = (torch.cat([get("shared.up"), get("shared.sg")], 0).to(device, dtype).contiguous(),
+                               get("shared.down").to(device, dtype).contiguous())
+            self.shared_limit = float(shared_limit or 0.0)
+
+    def route(self, h):
+        if self.routing == "grouped_softmax":
+            z = F.linear(h.float(), self.router)
+            return M.moe_topk(z, self.correction, self.top, self.groups, self.keep)
+        return M.moe_top_logits(F.linear(h.float(), self.router, self.router_bias), self.top)
+
+    def _act(self, u):
+        return M.clamp_swiglu(u, self.limit) if self.act == "clamp_glu" else M.relu_sq(u)
 
     def __call__(self, h, ctx=None) -> torch.Tensor:
         t, width = h.shape
         out = torch.zeros(t, width, dtype=torch.float32, device=h.device)
-        z = F.linear(h.float(), self.router)
-        idx, wts = M.moe_topk(z, self.correction, self.top, self.groups, self.keep)
+        idx, wts = self.route(h)
         if t <= self.PAIR_ROWS:
             # decode-size steps: per-pair weight streaming, nothing read back on the host
-            M.moe_pairs(out, h, idx, wts, self.wgu, self.wdown, self.limit)
+            M.moe_pairs(out, h, idx, wts, self.wgu, self.wdown, self.limit, self.act)
             return self._shared(out, h)
         flat = idx.view(-1).long()
         order = torch.argsort(flat, stable=True)
@@ -382,7 +457,7 @@ class MoEFF:
         for e, n in enumerate(counts):
             if n == 0:
                 continue
-            y = M.clamp_swiglu(F.linear(hs[a:a + n], self.wgu[e]), self.limit)
+            y = self._act(F.linear(hs[a:a + n], self.wgu[e]))
             M.scale_add_rows(out, F.linear(y, self.wdown[e]), rows[a:a + n], w[a:a + n])
             a += n
         return self._shared(out, h)
@@ -393,10 +468,13 @@ class MoEFF:
 
     def _shared(self, out, h):
         if self.shared is not None:
-            wgu, wdown = self.shared
-            gu = F.linear(h, wgu)
-            y = M.clamp_swiglu(gu, self.shared_limit)
-            M.scale_add_rows(out, F.linear(y, wdown), None, gu[:, -1].contiguous(), sigmoid=True)
+            w1, wdown = self.shared
+            u = F.linear(h, w1)
+            if self.act == "clamp_glu":
+                y = M.clamp_swiglu(u, self.shared_limit)
+            else:
+                y = M.relu_sq(u[:, :-1].contiguous())
+            M.scale_add_rows(out, F.linear(y, wdown), None, u[:, -1].contiguous(), sigmoid=True)
         return out
 
 

@@ -11,6 +11,12 @@ builds the layer list in ``load_tensors``.
 Per run, with x the residual:  x += norm1b(mixer(norm1 x));
 x += norm2b(ff(norm2 x)) (if the layer has a feed-forward);
 x += rms(side(x, token)) * side.norm (if it has a token-side input).
+
+A model with ``norm_style = "layer_post"`` has no norm in front of its sublayers: they
+read x itself, and a layer norm with weight and bias sits on each sublayer's output,
+x += ln1(mixer(x)); x += ln2(ff(x)); the embedding rows (plus, optionally, a sinusoidal
+position vector) pass a layer norm before the first layer, and the final norm is a layer
+norm too.
 """
 from __future__ import annotations
 
@@ -36,6 +42,9 @@ class StackedLayer:
     norm2b: Optional[torch.Tensor] = None
     ff: Optional[object] = None
     side: Optional[object] = None
+    # biases of the output norms (layer-norm models)
+    bias1: Optional[torch.Tensor] = None
+    bias2: Optional[torch.Tensor] = None
 
 
 class StackedCache:
@@ -54,6 +63,7 @@ class StackedModel:
     needs_state_slots = True     # the runner hands every sequence a state slot
     supports_graphs = True
     family = "stacked"
+    norm_style = "rms_pre_post"   # or "layer_post"
 
     def __init__(self, cfg, device, dtype=torch.bfloat16, comm: TPComm = SINGLE,
                  max_model_len: int = 8192, quantization: Optional[str] = None):
@@ -68,6 +78,10 @@ class StackedModel:
         self.layers: List[StackedLayer] = []
         self.embed = self.head = self.final_norm = self.loop_step = None
         self.embed_scale = 1.0
+        self.pos_freqs = None                   # fp32 sinusoid frequencies (position vector added to the embedding)
+        self.embed_norm = None                  # (weight, bias) of the layer norm after the embedding
+        self.final_bias = None
+        self.logit_softcap = 0.0
         self.vocab_pad = 0
         self.mark_at = None
         self.layer_tap: Optional[list] = None   # tests: fp32 residual after every layer run
@@ -156,6 +170,8 @@ class StackedModel:
         if seg is None:
             raise ValueError("this model needs the step's row segments (AttnMeta.segments)")
         ctx = StepContext(input_ids, meta.positions, meta.slot_mapping, seg)
+        if self.norm_style == "layer_post":
+            return self._forward_layer_post(input_ids, meta, ctx, caches)
         x = M.embed_rows(input_ids, self.embed, self.embed_scale)
         tap = self.layer_tap
         fuse_step = tap is None
@@ -196,10 +212,33 @@ class StackedModel:
             return rows.to(dt)
         return M.rms_norm_rows(rows, self.final_norm, eps, dt)
 
+    def _forward_layer_post(self, input_ids, meta, ctx, caches: StackedCache) -> torch.Tensor:
+        dt, eps = self.dtype, self.cfg.rms_norm_eps
+        x = M.embed_rows(input_ids, self.embed, self.embed_scale, meta.positions, self.pos_freqs)
+        h = M.add_layer_norm_rows(x, None, self.embed_norm[0], self.embed_norm[1], eps, dt) \
+            if self.embed_norm is not None else (x if dt == torch.float32 else x.to(dt))
+        tap, mark = self.layer_tap, self.mark_at
+        for r, (li, _) in enumerate(self.runs):
+            if mark is not None and r == mark[0]:
+                mark[1].record()
+            L = self.layers[li]
+            h = M.add_layer_norm_rows(x, L.mixer(h, ctx, caches.per_run[r]), L.norm1b, L.bias1, eps, dt)
+            if L.ff is not None:
+                h = M.add_layer_norm_rows(x, L.ff(h, ctx), L.norm2b, L.bias2, eps, dt)
+            if tap is not None:
+                tap.append(x.clone())
+        idx = meta.logits_indices
+        rows = x.index_select(0, idx) if idx.numel() != x.shape[0] else x
+        if rows.shape[0] == 0:
+            return rows.to(dt)
+        return M.layer_norm_rows(rows, self.final_norm, self.final_bias, eps, dt)
+
     def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
         """fp32 logits [rows, vocab rounded up to a multiple of 8]; columns past the
-        vocabulary are -inf."""
+        vocabulary are -inf.  With ``logit_softcap`` c > 0 the logits are c tanh(z / c)."""
         logits = self._head_product(h)
+        if self.logit_softcap:
+            M.tanh_cap_(logits, self.logit_softcap)
         if self.vocab_pad:
             logits[:, self.cfg.vocab_size:] = float("-inf")
         return logits

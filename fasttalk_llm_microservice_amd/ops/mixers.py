@@ -71,13 +71,52 @@ class Segments:
 # residual stream (fp32) and norms
 # ---------------------------------------------------------------------------------
 
-def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
-    """fp32 residual rows table[ids] * scale."""
+def embed_rows(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0,
+               positions: Optional[torch.Tensor] = None,
+               pos_freqs: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 residual rows table[ids] * scale; with ``pos_freqs`` (fp32 [ceil(width/2)],
+    :func:`sinusoid_freqs`) a sinusoidal position vector is added: column 2i gets
+    sin(p f_i), column 2i+1 cos(p f_i), angles in fp32."""
     if ids.is_cuda:
         out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32, device=ids.device)
-        native_mixers().embed_rows(out, ids, table, float(scale))
+        native_mixers().embed_rows(out, ids, table, float(scale), positions if pos_freqs is not None else None,
+                                   pos_freqs)
         return out
-    return ref.embed_rows(ids, table, scale)
+    return ref.embed_rows(ids, table, scale, positions, pos_freqs)
+
+
+sinusoid_freqs = ref.sinusoid_freqs
+
+
+def layer_norm_rows(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """(x - mean) / sqrt(var + eps) * w + b of fp32 rows x (var = mean squared deviation),
+    rounded to ``out_dtype``; x is left as it is."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        native_mixers().layer_norm(x, None, w, b, out, None, eps)
+        return out
+    return ref.layer_norm_rows(x, w, b, eps, out_dtype)
+
+
+def add_layer_norm_rows(residual: torch.Tensor, y: Optional[torch.Tensor], w: torch.Tensor, b: torch.Tensor,
+                        eps: float, out_dtype) -> torch.Tensor:
+    """residual (fp32, in place) += layer_norm(y) * w + b, or, without y, residual <-
+    layer_norm(residual) * w + b.  Returns the new residual in ``out_dtype`` (the residual
+    itself when that is fp32): what the next sublayer of a post-norm stack reads."""
+    if residual.is_cuda:
+        cast = None if out_dtype == torch.float32 else \
+            torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+        native_mixers().layer_norm(residual, y, w, b, None, cast, eps)
+        return residual if cast is None else cast
+    return ref.add_layer_norm_rows(residual, y, w, b, eps, out_dtype)
+
+
+def tanh_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """fp32 x <- cap * tanh(x / cap) in place; infinite entries stay as they are."""
+    if x.is_cuda:
+        native_mixers().tanh_cap(x, float(cap))
+        return x
+    return ref.tanh_cap_(x, cap)
 
 
 def rms_norm_rows(x: torch.Tensor, w: torch.Tensor, eps: float, out_dtype,
@@ -318,13 +357,35 @@ def attn_prep(qkv, nq: int, nk: int, q_norm_w, k_norm_w, eps: float, table, rot_
                          slot_mapping, k_cache, v_cache)
 
 
+def conv_attn_prep(qkv, nq: int, nk: int, conv_w, conv_state, seg: Segments, q_norm_w, k_norm_w, eps: float,
+                   head_dim: int, slot_mapping, k_cache, v_cache) -> torch.Tensor:
+    """Rows [q (nq) | k (nk) | v] of a fused projection pass a per-channel causal
+    convolution over time (``conv_w`` [C, taps] fp32, last column = the current row, no
+    bias, no activation; ``conv_state`` [slots, taps-1, C] fp32 holds each sequence's last
+    projected rows and is updated; a segment at position 0 starts from zeros), then every
+    ``head_dim`` chunk of q and of k is divided by its root mean square and multiplied by
+    ``q_norm_w`` / ``k_norm_w`` ([head_dim], shared by the heads; None: no norm).
+    Convolution and norm are fp32.  Returns fp32 queries [T, nq]; keys and values go to
+    the rows' cache slots."""
+    if qkv.is_cuda:
+        q = torch.empty(qkv.shape[0], nq, dtype=torch.float32, device=qkv.device)
+        native_mixers().conv_attn_prep(q, qkv, nq, nk, conv_w, conv_state, seg.start, seg.pos0, seg.slot, seg.num,
+                                       q_norm_w, k_norm_w, eps, head_dim, slot_mapping, k_cache, v_cache)
+        return q
+    return ref.conv_attn_prep(qkv, nq, nk, conv_w, conv_state, seg, q_norm_w, k_norm_w, eps, head_dim,
+                              slot_mapping, k_cache, v_cache)
+
+
 @dataclasses.dataclass
 class WindowSpec:
     """A windowed attention's constants.  Query head a = h * maps + m (head h, score map
     m) reads key head floor(h / (heads / kv_heads)) * maps + m and value head
     floor(h / (heads / kv_heads)).  Position i sees j iff 0 <= i - j < window (window 0:
-    every earlier key).  score = q.k * scale - r1[a] ln(1 + r2[a] (i - j)); weight =
-    softmax over the visible keys, or sigmoid(score + pb[a]) without normalisation."""
+    every earlier key).  s = q.k * scale; with ``softcap`` c > 0, s <- c tanh(s / c);
+    score = s - r1[a] ln(1 + r2[a] (i - j)); weight = softmax over the visible keys, or
+    sigmoid(score + pb[a]) without normalisation.  ``sink`` (a score, softmax only): the
+    softmax's denominator gains exp(sink), as if one more key with that score and no
+    value were always visible."""
     heads: int
     kv_heads: int
     dk: int
@@ -336,6 +397,8 @@ class WindowSpec:
     r1: Optional[torch.Tensor] = None     # fp32 [heads * maps] (with r2)
     r2: Optional[torch.Tensor] = None
     pb: Optional[torch.Tensor] = None     # fp32 [heads * maps] (sigmoid weights only)
+    softcap: float = 0.0
+    sink: Optional[float] = None
 
 
 def window_attention(q, k_cache, v_cache, seg: Segments, spec: WindowSpec, skip_from: int = 0,
@@ -350,10 +413,10 @@ def window_attention(q, k_cache, v_cache, seg: Segments, spec: WindowSpec, skip_
         native_mixers().window_attention(out, q, k_cache, v_cache, seg.start, seg.pos0, seg.kv_len,
                                          seg.block_tables, seg.num, seg.max_rows, sp.heads, sp.maps,
                                          sp.kv_heads, sp.dk, sp.dv, sp.window, sp.scale, sp.sigmoid,
-                                         sp.r1, sp.r2, sp.pb, skip_from)
+                                         sp.r1, sp.r2, sp.pb, skip_from, float(sp.softcap), sp.sink)
         return out
     r = ref.window_attention(q, k_cache, v_cache, seg, sp.heads, sp.maps, sp.kv_heads, sp.dk, sp.dv,
-                             sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb)
+                             sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, sp.softcap, sp.sink)
     if out is not None:
         out.copy_(r)
         return out
@@ -368,14 +431,16 @@ def band_weights(s, first_pos: int, key0: int, spec: WindowSpec, rep_rows: int):
     sp = spec
     if s.is_cuda:
         native_mixers().band_weights(s, rep_rows, first_pos, key0, sp.heads, sp.maps, sp.kv_heads,
-                                     sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb)
+                                     sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, float(sp.softcap),
+                                     sp.sink)
         return s
     g, rr, keys = s.shape
     rep = sp.heads // sp.kv_heads
     # [G, maps, rep, rows, keys] -> query-head order (g, r, m)
     v = s.view(sp.kv_heads, sp.maps, rep, rep_rows, keys).permute(0, 2, 1, 3, 4) \
         .reshape(sp.heads * sp.maps, rep_rows, keys)
-    w = ref.band_weights(v, first_pos, key0, sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb)
+    w = ref.band_weights(v, first_pos, key0, sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, sp.softcap,
+                         sp.sink)
     s.copy_(w.view(sp.kv_heads, rep, sp.maps, rep_rows, keys).permute(0, 2, 1, 3, 4).reshape(g, rr, keys))
     return s
 
@@ -458,14 +523,27 @@ def moe_topk(z, correction, top: int, groups: int, keep: int):
     return ref.moe_topk(z, correction, top, groups, keep)
 
 
-def moe_pairs(out, h, idx, wts, wgu, wdown, limit: float):
+def moe_top_logits(z, top: int):
+    """Router: the ``top`` largest logits of each fp32 row (ties to the lower index) and,
+    as weights, the softmax over just those."""
+    if z.is_cuda:
+        t = z.shape[0]
+        idx = torch.empty(t, top, dtype=torch.int32, device=z.device)
+        wts = torch.empty(t, top, dtype=torch.float32, device=z.device)
+        native_mixers().moe_top_logits(idx, wts, z, top)
+        return idx, wts
+    return ref.moe_top_logits(z, top)
+
+
+def moe_pairs(out, h, idx, wts, wgu, wdown, limit: float = 0.0, act: str = "clamp_glu"):
     """Few rows (decode): out (fp32, in place) += sum_k wts[:, k] * expert_{idx[:, k]}(h),
-    every (row, expert) pair streaming its expert's [gate | up] and down matrices; no
-    host round trip, so the step can be captured in a hipGraph."""
+    every (row, expert) pair streaming its expert's first matrix ([gate | up] with the
+    clamped GLU, ``act`` "clamp_glu"; or up alone with relu(.)^2, ``act`` "relu_sq") and
+    its down matrix; no host round trip, so the step can be captured in a hipGraph."""
     if out.is_cuda:
-        native_mixers().moe_pairs(out, h, idx, wts, wgu, wdown, float(limit))
+        native_mixers().moe_pairs(out, h, idx, wts, wgu, wdown, float(limit), act == "relu_sq")
     else:
-        ref.moe_pairs(out, h, idx, wts, wgu, wdown, limit)
+        ref.moe_pairs(out, h, idx, wts, wgu, wdown, limit, act)
 
 
 def clamp_swiglu(gu, limit: float):

@@ -14,9 +14,49 @@ import torch
 import torch.nn.functional as F
 
 
-def embed_rows(ids, table, scale=1.0):
+def embed_rows(ids, table, scale=1.0, positions=None, pos_freqs=None):
     x = table.index_select(0, ids.long()).float()
-    return x * scale if scale != 1.0 else x
+    x = x * scale if scale != 1.0 else x
+    if pos_freqs is not None:
+        x = x + sinusoid_rows(positions[:ids.shape[0]], pos_freqs, x.shape[1])
+    return x
+
+
+def sinusoid_freqs(width: int, base: float = 10000.0, device=None):
+    """fp32 [ceil(width / 2)]: f_i = base^(-2i/width), evaluated in double precision."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / width)).float().to(device)
+
+
+def sinusoid_rows(positions, freqs, width: int):
+    """fp32 [T, width]: column 2i = sin(p f_i), column 2i+1 = cos(p f_i) (fp32 angles)."""
+    a = positions.float()[:, None] * freqs.float()[None]
+    return torch.stack([a.sin(), a.cos()], -1).reshape(positions.shape[0], -1)[:, :width]
+
+
+def _layer_norm(x, w, b, eps):
+    mu = x.mean(-1, keepdim=True)
+    d = x - mu
+    return d * torch.rsqrt((d * d).mean(-1, keepdim=True) + eps) * w.float() + b.float()
+
+
+def layer_norm_rows(x, w, b, eps, out_dtype):
+    return _layer_norm(x.float(), w, b, eps).to(out_dtype)
+
+
+def add_layer_norm_rows(residual, y, w, b, eps, out_dtype):
+    if y is None:
+        residual.copy_(_layer_norm(residual, w, b, eps))
+    else:
+        residual.add_(_layer_norm(y.float(), w, b, eps))
+    return residual if out_dtype == torch.float32 else residual.to(out_dtype)
+
+
+def tanh_cap_(x, cap: float):
+    """x <- cap * tanh(x / cap) in place (fp32); infinite entries (masked columns) stay."""
+    fin = torch.isfinite(x)
+    x.copy_(torch.where(fin, cap * torch.tanh(x / cap), x))
+    return x
 
 
 def _rms(x, eps):
@@ -198,11 +238,19 @@ def moe_topk(z, correction, top, groups, keep):
     return idx.int(), s.gather(1, idx)
 
 
-def moe_pairs(out, h, idx, wts, wgu, wdown, limit):
+def moe_top_logits(z, top):
+    """The ``top`` largest logits per row (ties to the lower index) and the softmax over
+    just those."""
+    val, idx = torch.sort(z.float(), dim=-1, descending=True, stable=True)
+    return idx[:, :top].int(), torch.softmax(val[:, :top], -1)
+
+
+def moe_pairs(out, h, idx, wts, wgu, wdown, limit, act="clamp_glu"):
     for t in range(h.shape[0]):
         for k in range(idx.shape[1]):
             e = int(idx[t, k])
-            y = clamp_swiglu(F.linear(h[t:t + 1], wgu[e]), limit)
+            u = F.linear(h[t:t + 1], wgu[e])
+            y = clamp_swiglu(u, limit) if act == "clamp_glu" else relu_sq(u)
             out[t] += wts[t, k] * F.linear(y, wdown[e])[0].float()
 
 
@@ -265,7 +313,38 @@ def attn_prep(qkv, nq, nk, q_norm_w, k_norm_w, eps, table, rot_dims, head_dim, p
     return q.contiguous()
 
 
-def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb):
+def conv_attn_prep(qkv, nq, nk, conv_w, conv_state, seg, q_norm_w, k_norm_w, eps, head_dim, slot_mapping,
+                   k_cache, v_cache):
+    t = qkv.shape[0]
+    taps = conv_w.shape[1]
+    w = conv_w.float()
+    y = torch.zeros(qkv.shape, dtype=torch.float32, device=qkv.device)
+    start = seg.start.tolist()
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        slot = int(seg.slot[s])
+        if slot < 0 or b == a:
+            continue
+        hist = conv_state[slot] if int(seg.pos0[s]) > 0 else torch.zeros_like(conv_state[slot])
+        xp = torch.cat([hist, qkv[a:b].float()], 0)
+        n = b - a
+        y[a:b] = sum(xp[j:j + n] * w[:, j][None] for j in range(taps))
+        if taps > 1:
+            conv_state[slot] = xp[n:]
+    q, k, v = y[:, :nq], y[:, nq:nq + nk], y[:, nq + nk:]
+    if q_norm_w is not None:
+        q = (_rms(q.reshape(t, -1, head_dim), eps) * q_norm_w.float()).reshape(t, nq)
+    if k_norm_w is not None:
+        k = (_rms(k.reshape(t, -1, head_dim), eps) * k_norm_w.float()).reshape(t, nk)
+    slots = slot_mapping[:t].long()
+    keep = slots >= 0
+    if keep.any():
+        k_cache.view(-1, k_cache.shape[-1])[slots[keep]] = k[keep].to(k_cache.dtype)
+        v_cache.view(-1, v_cache.shape[-1])[slots[keep]] = v[keep].to(v_cache.dtype)
+    return q.contiguous()
+
+
+def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb, softcap=0.0, sink=None):
     """s fp32 [heads, rows, keys] raw dot products -> attention weights: row r is position
     first_pos + r, column c is position key0 + c, visible iff 0 <= i - j (< window)."""
     heads, rows, keys = s.shape
@@ -275,6 +354,8 @@ def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb):
     if window > 0:
         vis &= dist < window
     z = s * scale
+    if softcap:
+        z = softcap * torch.tanh(z / softcap)
     if r1 is not None:
         z = z - r1.float()[:, None, None] * torch.log(1.0 + r2.float()[:, None, None]
                                                       * dist.clamp_min(0).float()[None])
@@ -283,11 +364,15 @@ def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb):
             z = z + pb.float()[:, None, None]
         return torch.sigmoid(z) * vis[None]
     z = z.masked_fill(~vis[None], float("-inf"))
+    if sink is not None:
+        m = z.max(-1, keepdim=True).values.clamp_min(float(sink))
+        e = torch.exp(z - m)
+        return e / (torch.exp(float(sink) - m) + e.sum(-1, keepdim=True))
     return torch.softmax(z, -1).masked_fill(~vis[None], 0.0)
 
 
 def window_attention(q, k_cache, v_cache, seg, heads, maps, kv_heads, dk, dv, window, scale, sigmoid,
-                     r1, r2, pb):
+                     r1, r2, pb, softcap=0.0, sink=None):
     """q fp32 [T, heads*maps*dk]; caches [blocks, bs, kv_heads*maps*dk] / [blocks, bs,
     kv_heads*dv]; returns fp32 [T, heads*maps, dv]."""
     t = q.shape[0]
@@ -312,7 +397,7 @@ def window_attention(q, k_cache, v_cache, seg, heads, maps, kv_heads, dk, dv, wi
         v = v_cache[blocks].reshape(nblk * bs, -1)[lo:n].float().view(n - lo, kv_heads, dv)
         qs = q[a:b].view(b - a, hq, dk)
         sc = torch.einsum("thd,jhd->htj", qs, k[:, khead])
-        w = band_weights(sc, p0, lo, window, scale, sigmoid, r1, r2, pb)
+        w = band_weights(sc, p0, lo, window, scale, sigmoid, r1, r2, pb, softcap, sink)
         out[a:b] = torch.einsum("htj,jhd->thd", w, v[:, vhead])
     return out
 
