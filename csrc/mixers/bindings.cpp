@@ -11,7 +11,16 @@
 
 extern "C" {
 int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows, int width, int vocab,
-                  float scale, hipStream_t s);
+                  float scale, const int* positions, const float* freqs, hipStream_t s);
+int mx_layer_norm(float* x, const void* y, int y_bf16, long y_stride, const float* w, const float* b, void* out,
+                  void* cast, int out_bf16, int rows, int width, float eps, hipStream_t s);
+int mx_tanh_cap(float* x, long n, float cap, hipStream_t s);
+int mx_conv_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv,
+                      const float* conv_w, int taps, float* hist, const int* start, const int* pos0, const int* slot,
+                      int num_segs, int num_state_slots, const float* wq, const float* wk, float eps, int head_dim,
+                      const int* slots, void* k_cache, void* v_cache, int cache_bf16, long num_slots, long rows,
+                      hipStream_t s);
+int mx_moe_top_logits(int* idx, float* wts, const float* z, long rows, int experts, int top, hipStream_t s);
 int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, hipStream_t s);
 int mx_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv, const float* wq,
                  const float* wk, float eps, const float* table, int table_rows, int rot_dims, int head_dim,
@@ -22,10 +31,10 @@ int mx_window_attention(float* out, const float* q, const void* k_cache, const v
                         const int* start, const int* pos0, const int* kv_len, const int* bt, int bt_stride,
                         int num_segs, long total_rows, int heads, int maps, int kv_heads, int dk, int dv, int window,
                         float scale, int sigmoid, const float* r1, const float* r2, const float* pb, int block_size,
-                        int num_blocks, int skip_from, hipStream_t s);
+                        int num_blocks, int skip_from, float softcap, int has_sink, float sink, hipStream_t s);
 int mx_band_weights(float* S, int gk, int rep_rows_total, int rows, int keys, int first_pos, int key0, int heads,
                     int maps, int kv_heads, int window, float scale, int sigmoid, const float* r1, const float* r2,
-                    const float* pb, hipStream_t s);
+                    const float* pb, float softcap, int has_sink, float sink, hipStream_t s);
 int mx_diff_combine(void* out, int out_bf16, const float* a, const void* gate, int gate_bf16, long gate_stride,
                     long rows, int heads, int dv, float lam, float post, float eps, hipStream_t s);
 int mx_ssd_max_state();
@@ -79,7 +88,7 @@ int mx_causal_softmax(void* P, int p_bf16, const float* S, long rows, int rows_p
                       float scale, hipStream_t s);
 int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h_stride, const int* idx, const float* wts,
                  const void* wgu, const void* wdown, long rows, int top, int experts, int ff, int width,
-                 float limit, hipStream_t s);
+                 float limit, int relu_sq, hipStream_t s);
 int mx_moe_topk(int* idx, float* wts, const float* z, const float* corr, long rows, int experts, int top,
                 int groups, int keep, hipStream_t s);
 }
@@ -116,13 +125,61 @@ void check_segs(const Tensor& start, const Tensor& a, const Tensor& b, int64_t n
   TORCH_CHECK(num >= 0 && start.numel() >= num + 1 && a.numel() >= num && b.numel() >= num, "segment arrays too short");
 }
 
-void embed_rows(Tensor out, Tensor ids, Tensor table, double scale) {
+void embed_rows(Tensor out, Tensor ids, Tensor table, double scale, OptT positions, OptT freqs) {
   check_f32(out, "out");
   check_i32(ids, "ids");
   TORCH_CHECK(table.is_cuda() && is_act(table) && table.is_contiguous() && table.dim() == 2, "table");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == ids.numel() && out.size(1) == table.size(1), "out shape");
+  const int* pp = nullptr;
+  const float* fp = nullptr;
+  if (freqs) {
+    TORCH_CHECK(positions, "positions go with the sinusoid frequencies");
+    check_i32(*positions, "positions");
+    check_f32(*freqs, "sinusoid frequencies");
+    TORCH_CHECK(positions->numel() >= ids.numel() && freqs->numel() * 2 >= table.size(1), "positions / frequencies size");
+    pp = positions->data_ptr<int>();
+    fp = freqs->data_ptr<float>();
+  }
   chk(mx_embed_rows(out.data_ptr<float>(), ids.data_ptr<int>(), table.data_ptr(), bf(table), (int)ids.numel(),
-                    (int)table.size(1), (int)table.size(0), (float)scale, stream()), "embed_rows");
+                    (int)table.size(1), (int)table.size(0), (float)scale, pp, fp, stream()), "embed_rows");
+}
+
+// x (fp32 residual) with y: x += ln(y), cast = x; without y: out = ln(x), or, without out, x = ln(x), cast = x
+void layer_norm(Tensor x, OptT y, Tensor w, Tensor b, OptT out, OptT cast, double eps) {
+  check_f32(x, "residual");
+  TORCH_CHECK(x.dim() == 2, "residual 2-D");
+  const int64_t rows = x.size(0), width = x.size(1);
+  check_f32(w, "norm weight");
+  check_f32(b, "norm bias");
+  TORCH_CHECK(w.numel() == width && b.numel() == width, "norm weight / bias size");
+  TORCH_CHECK(!(y && out), "out goes without y");
+  const void* yp = nullptr;
+  int ybf = 0;
+  long ys = 0;
+  if (y) {
+    check_rows(*y, "y");
+    TORCH_CHECK(y->size(0) == rows && y->size(1) == width, "y shape");
+    yp = y->data_ptr();
+    ybf = bf(*y);
+    ys = y->stride(0);
+  }
+  int obf = 0;
+  void *op = nullptr, *cp = nullptr;
+  for (const OptT* t : {&out, &cast}) {
+    if (!*t) continue;
+    TORCH_CHECK((*t)->is_cuda() && (*t)->is_contiguous() && is_act(**t) && (*t)->sizes() == x.sizes(), "out / cast");
+    obf = bf(**t);
+  }
+  if (out) op = out->data_ptr();
+  if (cast) cp = cast->data_ptr();
+  chk(mx_layer_norm(x.data_ptr<float>(), yp, ybf, ys, w.data_ptr<float>(), b.data_ptr<float>(), op, cp, obf,
+                    (int)rows, (int)width, (float)eps, stream()), "layer_norm");
+}
+
+void tanh_cap(Tensor x, double cap) {
+  check_f32(x, "x");
+  TORCH_CHECK(cap > 0, "cap > 0");
+  chk(mx_tanh_cap(x.data_ptr<float>(), x.numel(), (float)cap, stream()), "tanh_cap");
 }
 
 void add_rms_norm(Tensor x, OptT y, OptT wb, OptT add_vec, OptT next_w, OptT out, OptT cast, double eps) {
@@ -357,7 +414,18 @@ void moe_topk(Tensor idx, Tensor wts, Tensor z, Tensor corr, int64_t top, int64_
                   z.size(0), (int)z.size(1), (int)top, (int)groups, (int)keep, stream()), "moe_topk");
 }
 
-void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor wdown, double limit) {
+void moe_top_logits(Tensor idx, Tensor wts, Tensor z, int64_t top) {
+  check_i32(idx, "idx");
+  check_f32(wts, "wts");
+  check_f32(z, "z");
+  TORCH_CHECK(z.dim() == 2 && top >= 1 && top <= z.size(1) && idx.numel() == z.size(0) * top &&
+              wts.numel() == z.size(0) * top, "moe_top_logits shapes");
+  chk(mx_moe_top_logits(idx.data_ptr<int>(), wts.data_ptr<float>(), z.data_ptr<float>(), z.size(0), (int)z.size(1),
+                        (int)top, stream()), "moe_top_logits");
+}
+
+// relu_sq: the experts' first matrix is [ff, width] (up alone) instead of [2 ff, width] (gate | up)
+void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor wdown, double limit, bool relu_sq) {
   check_f32(out, "out");
   check_rows(h, "h");
   check_i32(idx, "idx");
@@ -365,17 +433,18 @@ void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor 
   TORCH_CHECK(wgu.is_cuda() && wgu.is_contiguous() && wgu.dim() == 3 && wdown.is_cuda() && wdown.is_contiguous() &&
               wdown.dim() == 3 && wgu.scalar_type() == h.scalar_type() && wdown.scalar_type() == h.scalar_type(),
               "expert weights");
-  const int64_t rows = h.size(0), width = h.size(1), experts = wgu.size(0), ff = wgu.size(1) / 2;
+  const int64_t rows = h.size(0), width = h.size(1), experts = wgu.size(0);
+  const int64_t ff = relu_sq ? wgu.size(1) : wgu.size(1) / 2;
   TORCH_CHECK(idx.dim() == 2 && idx.size(0) == rows && wts.sizes() == idx.sizes(), "idx / wts");
   const int64_t top = idx.size(1);
   TORCH_CHECK(wgu.size(2) == width && wdown.size(0) == experts && wdown.size(1) == width && wdown.size(2) == ff &&
-              wgu.size(1) == 2 * ff && out.dim() == 2 && out.size(0) == rows && out.size(1) == width,
+              wgu.size(1) == (relu_sq ? ff : 2 * ff) && out.dim() == 2 && out.size(0) == rows && out.size(1) == width,
               "moe_pairs shapes");
   TORCH_CHECK(((uintptr_t)h.data_ptr()) % 16 == 0, "h alignment");
   Tensor y = at::empty({rows * top, ff}, h.options());
   chk(mx_moe_pairs(out.data_ptr<float>(), y.data_ptr(), h.data_ptr(), bf(h), h.stride(0), idx.data_ptr<int>(),
                    wts.data_ptr<float>(), wgu.data_ptr(), wdown.data_ptr(), rows, (int)top, (int)experts, (int)ff,
-                   (int)width, (float)limit, stream()), "moe_pairs");
+                   (int)width, (float)limit, relu_sq ? 1 : 0, stream()), "moe_pairs");
 }
 
 void gelu_glu(Tensor out, Tensor gu) {
@@ -427,10 +496,37 @@ void attn_prep(Tensor q, Tensor qkv, int64_t nq, int64_t nk, OptT wq, OptT wk, d
                    v_cache.data_ptr(), bf(k_cache), k_cache.size(0) * k_cache.size(1), t, stream()), "attn_prep");
 }
 
+void conv_attn_prep(Tensor q, Tensor qkv, int64_t nq, int64_t nk, Tensor conv_w, Tensor hist, Tensor start,
+                    Tensor pos0, Tensor slot, int64_t num_segs, OptT wq, OptT wk, double eps, int64_t head_dim,
+                    Tensor slots, Tensor k_cache, Tensor v_cache) {
+  check_f32(q, "q");
+  check_rows(qkv, "qkv");
+  check_i32(slots, "slot_mapping");
+  check_f32(conv_w, "conv_w");
+  check_f32(hist, "conv_state");
+  const int64_t t = qkv.size(0), c = qkv.size(1), nv = c - nq - nk;
+  TORCH_CHECK(nq >= 1 && nk >= 1 && nv >= 1 && head_dim >= 1 && nq % head_dim == 0 && nk % head_dim == 0 &&
+              q.numel() == t * nq && slots.numel() >= t, "conv_attn_prep shapes");
+  const int64_t taps = conv_w.dim() == 2 ? conv_w.size(1) : 0;
+  TORCH_CHECK(conv_w.dim() == 2 && conv_w.size(0) == c && taps >= 1 && taps <= 16 && hist.dim() == 3 &&
+              hist.size(1) == taps - 1 && hist.size(2) == c, "conv shapes");
+  check_segs(start, pos0, slot, num_segs);
+  check_cache(k_cache, nk, "k_cache");
+  check_cache(v_cache, nv, "v_cache");
+  TORCH_CHECK(k_cache.scalar_type() == v_cache.scalar_type() && k_cache.size(0) == v_cache.size(0) &&
+              k_cache.size(1) == v_cache.size(1), "k / v caches differ");
+  chk(mx_conv_attn_prep(q.data_ptr<float>(), qkv.data_ptr(), bf(qkv), qkv.stride(0), (int)nq, (int)nk, (int)nv,
+                        conv_w.data_ptr<float>(), (int)taps, hist.data_ptr<float>(), start.data_ptr<int>(),
+                        pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs, (int)hist.size(0),
+                        opt_f32(wq, head_dim, "q norm"), opt_f32(wk, head_dim, "k norm"), (float)eps, (int)head_dim,
+                        slots.data_ptr<int>(), k_cache.data_ptr(), v_cache.data_ptr(), bf(k_cache),
+                        k_cache.size(0) * k_cache.size(1), t, stream()), "conv_attn_prep");
+}
+
 void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor start, Tensor pos0, Tensor kv_len,
                       Tensor bt, int64_t num_segs, int64_t max_rows, int64_t heads, int64_t maps, int64_t kv_heads,
                       int64_t dk, int64_t dv, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb,
-                      int64_t skip_from) {
+                      int64_t skip_from, double softcap, c10::optional<double> sink) {
   check_f32(out, "out");
   check_f32(q, "q");
   TORCH_CHECK(heads >= 1 && maps >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && dk >= 1 && dv >= 1 &&
@@ -450,11 +546,13 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tens
                           bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, t, (int)heads, (int)maps, (int)kv_heads,
                           (int)dk, (int)dv, (int)window, (float)scale, sigmoid ? 1 : 0, opt_f32(r1, hq, "r1"),
                           opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), (int)k_cache.size(1), (int)k_cache.size(0),
-                          (int)skip_from, stream()), "window_attention");
+                          (int)skip_from, (float)softcap, sink ? 1 : 0, sink ? (float)*sink : 0.f, stream()),
+      "window_attention");
 }
 
 void band_weights(Tensor S, int64_t rows, int64_t first_pos, int64_t key0, int64_t heads, int64_t maps,
-                  int64_t kv_heads, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb) {
+                  int64_t kv_heads, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb,
+                  double softcap, c10::optional<double> sink) {
   check_f32(S, "S");
   TORCH_CHECK(S.dim() == 3 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && maps >= 1 &&
               S.size(0) == kv_heads * maps && rows >= 1 && S.size(1) == heads / kv_heads * rows && first_pos >= 0 &&
@@ -463,7 +561,8 @@ void band_weights(Tensor S, int64_t rows, int64_t first_pos, int64_t key0, int64
   const int64_t hq = heads * maps;
   chk(mx_band_weights(S.data_ptr<float>(), (int)S.size(0), (int)S.size(1), (int)rows, (int)S.size(2), (int)first_pos,
                       (int)key0, (int)heads, (int)maps, (int)kv_heads, (int)window, (float)scale, sigmoid ? 1 : 0,
-                      opt_f32(r1, hq, "r1"), opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), stream()), "band_weights");
+                      opt_f32(r1, hq, "r1"), opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), (float)softcap, sink ? 1 : 0,
+                      sink ? (float)*sink : 0.f, stream()), "band_weights");
 }
 
 void diff_combine(Tensor out, Tensor a, Tensor gate, double lam, double post, double eps, int64_t heads, int64_t dv) {
@@ -519,6 +618,10 @@ void gate_group_norm(Tensor out, Tensor y, Tensor z, Tensor w, double eps, int64
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_rows", &embed_rows);
   m.def("add_rms_norm", &add_rms_norm);
+  m.def("layer_norm", &layer_norm);
+  m.def("tanh_cap", &tanh_cap);
+  m.def("conv_attn_prep", &conv_attn_prep);
+  m.def("moe_top_logits", &moe_top_logits);
   m.def("head_rms_gate", &head_rms_gate);
   m.def("relu_sq", &relu_sq);
   m.def("clamp_swiglu", &clamp_swiglu);

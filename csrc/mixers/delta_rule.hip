@@ -288,6 +288,17 @@ extern "C" int mx_short_conv_silu(void* out, const void* x, int bf16, long x_str
   return (int)hipGetLastError();
 }
 
+// history update alone, for kernels that fuse the convolution into a larger step
+extern "C" int mx_conv_hist(const void* x, int bf16, long x_stride, float* hist, const int* start, const int* pos0,
+                            const int* slot, int num_segs, int channels, int taps, int num_slots, hipStream_t s) {
+  if (num_segs <= 0 || channels <= 0 || taps <= 1) return 0;
+  if (taps > kMaxTaps || num_segs > 65535) return -1;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((conv_hist_kernel<T>), dim3((channels + 255) / 256, num_segs), dim3(256),
+                                         0, s, (const T*)x, x_stride, hist, start, pos0, slot, channels, taps,
+                                         num_slots));
+  return (int)hipGetLastError();
+}
+
 extern "C" int mx_delta_prep(float* qn, float* kn, float* g, float* beta, const void* qkv, int bf16,
                              long qkv_stride, const void* a, long a_stride, const void* b, long b_stride,
                              const float* a_log, const float* dt_bias, long rows, int heads, int kv_heads,

@@ -2,6 +2,7 @@
 // back on the host): every (row, chosen expert) pair streams its expert's weights.
 //
 //   moe_gu_pairs:   y[pair, c] = glu(W_gate[e] h, W_up[e] h)[c]      (clamped GLU fused)
+//                   or, for experts without a gate, y[pair, c] = relu(W_up[e] h)[c]^2
 //   moe_down_pairs: out[row, c] += sum_k w[row, k] * (W_down[e_k] y[row, k])[c]   (fp32)
 //
 // One wave per output column, lanes along the reduction axis with 16-byte loads where
@@ -49,7 +50,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_gu_pairs_kernel(T* __restrict__ y, const T* __restrict__ h, long h_stride, const int* __restrict__ idx,
                     const T* __restrict__ wgu, int top, int experts, int ff, int width, float limit,
-                    int vec) {
+                    int vec, int relu_sq) {
   const int pair = blockIdx.y;
   const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (c >= ff) return;
@@ -57,6 +58,17 @@ moe_gu_pairs_kernel(T* __restrict__ y, const T* __restrict__ h, long h_stride, c
   int e = idx[pair];
   if (e < 0 || e >= experts) e = 0;
   const T* hr = h + (long)(pair / top) * h_stride;
+  if (relu_sq) {
+    // one matrix [ff, width] per expert
+    const float u0 = ft::wave_sum(dot_part(hr, wgu + ((long)e * ff + c) * width, width, lane, vec));
+    if (lane == 0) {
+      T tmp[1];
+      st(tmp, 0, u0);
+      const float u = fmaxf(ld(tmp, 0), 0.f);
+      st(y, (long)pair * ff + c, u * u);
+    }
+    return;
+  }
   const T* wg = wgu + ((long)e * 2 * ff + c) * width;
   const T* wu = wg + (long)ff * width;
   const float g0 = ft::wave_sum(dot_part(hr, wg, width, lane, vec));
@@ -101,7 +113,7 @@ using namespace mx;
 
 extern "C" int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h_stride, const int* idx,
                             const float* wts, const void* wgu, const void* wdown, long rows, int top,
-                            int experts, int ff, int width, float limit, hipStream_t s) {
+                            int experts, int ff, int width, float limit, int relu_sq, hipStream_t s) {
   if (rows <= 0) return 0;
   const long pairs = rows * top;
   if (pairs > 65535 || rows > 65535) return -1;
@@ -110,7 +122,7 @@ extern "C" int mx_moe_pairs(float* out, void* y, const void* h, int bf16, long h
   const int vec_dn = (ff % n == 0) ? 1 : 0;
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((moe_gu_pairs_kernel<T>), dim3((ff + 3) / 4, (unsigned)pairs), dim3(256),
                                          0, s, (T*)y, (const T*)h, h_stride, idx, (const T*)wgu, top, experts, ff,
-                                         width, limit, vec_gu));
+                                         width, limit, vec_gu, relu_sq));
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((moe_down_pairs_kernel<T>), dim3((width + 3) / 4, (unsigned)rows),
                                          dim3(256), 0, s, out, (const T*)y, idx, wts, (const T*)wdown, top,
                                          experts, ff, width, vec_dn));

@@ -4,7 +4,8 @@
 // is its best biased score; excluded experts count as -infinity), then the `top`
 // eligible experts with the largest biased scores.  Weights = the chosen experts'
 // unbiased softmax scores, not renormalised.  One wave per token; ties go to the lower
-// index.
+// index.  A second router (moe_top_logits) chooses on the logits and renormalises over
+// the chosen ones.
 #include "mx_common.h"
 
 namespace mx {
@@ -90,7 +91,48 @@ moe_topk_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __r
   }
 }
 
+// Routing on the logits themselves: the `top` largest logits of a row are chosen (ties to
+// the lower index) and weighted by the softmax over just those.  One wave per token.
+__global__ void __launch_bounds__(64)
+moe_top_logits_kernel(int* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ z, int experts,
+                      int top) {
+  extern __shared__ float sm[];
+  float* ch = sm;                   // logits, -inf once taken
+  float* val = sm + experts;        // the chosen logits, largest first
+  const long row = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* zr = z + row * experts;
+  for (int e = lane; e < experts; e += 64) ch[e] = zr[e];
+  __syncthreads();
+  for (int k = 0; k < top; ++k) {
+    Best b{-INFINITY, 1 << 30};
+    for (int e = lane; e < experts; e += 64) b = better(b, Best{ch[e], e});
+    b = wave_best(b);
+    const int e = b.i < experts ? b.i : 0;
+    if (lane == 0) {
+      idx[row * top + k] = e;
+      val[k] = b.v;
+      ch[e] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  float sum = 0.f;
+  for (int k = lane; k < top; k += 64) sum += expf(val[k] - val[0]);
+  sum = ft::wave_sum(sum);
+  for (int k = lane; k < top; k += 64) wts[row * top + k] = expf(val[k] - val[0]) / sum;
+}
+
 }  // namespace mx
+
+extern "C" int mx_moe_top_logits(int* idx, float* wts, const float* z, long rows, int experts, int top,
+                                 hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (experts < 1 || top < 1 || top > experts) return -1;
+  const size_t lds = (size_t)(experts + top) * sizeof(float);
+  if (lds > 60 * 1024) return -2;
+  hipLaunchKernelGGL(mx::moe_top_logits_kernel, dim3((unsigned)rows), dim3(64), lds, s, idx, wts, z, experts, top);
+  return (int)hipGetLastError();
+}
 
 extern "C" int mx_moe_topk(int* idx, float* wts, const float* z, const float* corr, long rows, int experts,
                            int top, int groups, int keep, hipStream_t s) {

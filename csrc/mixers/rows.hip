@@ -1,19 +1,74 @@
-// Row-wise kernels around an fp32 residual stream: embedding rows, the fused
-// "post-norm add + next pre-norm" step, per-head gated output norm, activations
+// Row-wise kernels around an fp32 residual stream: embedding rows (optionally with a
+// sinusoidal position vector), the fused "post-norm add + next pre-norm" step, the layer
+// norm (weight and bias) that adds a sublayer's output to the residual, the tanh cap of
+// the logits, per-head gated output norm, activations
 // (relu^2, clamped GLU, gelu GLU, gelu * token-side embedding) and the weighted row scatter-add
 // that combines expert outputs.
 #include "mx_common.h"
 
 namespace mx {
 
+// out = table[id] * scale (+ a sinusoidal position vector when freqs is given: column 2i
+// gets sin(p f_i), column 2i+1 cos(p f_i), with the angle p f_i formed in fp32)
 template <typename T>
 __global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict__ ids,
-                                  const T* __restrict__ table, int width, int vocab, float scale) {
+                                  const T* __restrict__ table, int width, int vocab, float scale,
+                                  const int* __restrict__ positions, const float* __restrict__ freqs) {
   const int row = blockIdx.x;
   int id = ids[row];
   if (id < 0 || id >= vocab) id = 0;
-  for (int i = threadIdx.x; i < width; i += blockDim.x)
-    out[(long)row * width + i] = ld(table, (long)id * width + i) * scale;
+  const float p = freqs != nullptr ? (float)positions[row] : 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = ld(table, (long)id * width + i) * scale;
+    if (freqs != nullptr) {
+      const float a = p * freqs[i >> 1];
+      v += (i & 1) ? cosf(a) : sinf(a);
+    }
+    out[(long)row * width + i] = v;
+  }
+}
+
+// layer norm with weight and bias, ln(u) = (u - mean) / sqrt(var + eps) * w + b with var
+// the mean squared deviation (two passes), around an fp32 residual x:
+//   y given:            x += ln(y);  cast = x
+//   y null, out null:   x  = ln(x);  cast = x
+//   y null, out given:  out = ln(x)  (x untouched)
+template <typename TY, typename TO, int NT>
+__global__ void layer_norm_kernel(float* __restrict__ x, const TY* __restrict__ y, long y_stride,
+                                  const float* __restrict__ w, const float* __restrict__ b,
+                                  TO* __restrict__ out, TO* __restrict__ cast, int width, float eps) {
+  __shared__ float red[NT / 64];
+  const long row = blockIdx.x;
+  float* xr = x + row * width;
+  const TY* yr = y != nullptr ? y + row * y_stride : nullptr;
+  auto src = [&](int i) { return yr != nullptr ? ld(yr, i) : xr[i]; };
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) sum += src(i);
+  const float mean = block_sum<NT>(sum, red) / (float)width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) {
+    const float d = src(i) - mean;
+    ss += d * d;
+  }
+  const float r = 1.0f / sqrtf(block_sum<NT>(ss, red) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += NT) {
+    const float v = (src(i) - mean) * r * w[i] + b[i];
+    if (out != nullptr) {
+      st(out, row * width + i, v);
+    } else {
+      const float nx = yr != nullptr ? xr[i] + v : v;
+      xr[i] = nx;
+      if (cast != nullptr) st(cast, row * width + i, nx);
+    }
+  }
+}
+
+// x <- cap * tanh(x / cap); infinite entries stay
+__global__ void tanh_cap_kernel(float* __restrict__ x, long n, float cap) {
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const float v = x[i];
+    if (isfinite(v)) x[i] = cap * tanhf(v / cap);
+  }
 }
 
 // residual (fp32, in place): x += rms_norm(y) * wb (+ add_vec);
@@ -150,10 +205,33 @@ __global__ void scale_add_rows_kernel(float* __restrict__ out, const TY* __restr
 using namespace mx;
 
 extern "C" int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int rows,
-                             int width, int vocab, float scale, hipStream_t s) {
+                             int width, int vocab, float scale, const int* positions, const float* freqs,
+                             hipStream_t s) {
   if (rows <= 0) return 0;
+  if (freqs != nullptr && positions == nullptr) return -1;
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((embed_rows_kernel<T>), dim3(rows), dim3(256), 0, s, out, ids,
-                                         (const T*)table, width, vocab, scale));
+                                         (const T*)table, width, vocab, scale, positions, freqs));
+  return (int)hipGetLastError();
+}
+
+template <typename TY, typename TO>
+static void launch_layer_norm(float* x, const void* y, long ys, const float* w, const float* b, void* out,
+                              void* cast, int rows, int width, float eps, hipStream_t s) {
+  hipLaunchKernelGGL((layer_norm_kernel<TY, TO, 256>), dim3(rows), dim3(256), 0, s, x, (const TY*)y, ys, w, b,
+                     (TO*)out, (TO*)cast, width, eps);
+}
+
+extern "C" int mx_layer_norm(float* x, const void* y, int y_bf16, long y_stride, const float* w, const float* b,
+                             void* out, void* cast, int out_bf16, int rows, int width, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (y != nullptr && out != nullptr) return -1;
+  if (y_bf16) {
+    if (out_bf16) launch_layer_norm<bf16_t, bf16_t>(x, y, y_stride, w, b, out, cast, rows, width, eps, s);
+    else launch_layer_norm<bf16_t, float>(x, y, y_stride, w, b, out, cast, rows, width, eps, s);
+  } else {
+    if (out_bf16) launch_layer_norm<float, bf16_t>(x, y, y_stride, w, b, out, cast, rows, width, eps, s);
+    else launch_layer_norm<float, float>(x, y, y_stride, w, b, out, cast, rows, width, eps, s);
+  }
   return (int)hipGetLastError();
 }
 
@@ -199,6 +277,13 @@ extern "C" int mx_head_rms_gate(void* out, int out_bf16, const float* o, const f
 static inline unsigned ew_grid(long n) {
   long g = (n + 255) / 256;
   return (unsigned)(g < 1 ? 1 : g > 65535 ? 65535 : g);
+}
+
+extern "C" int mx_tanh_cap(float* x, long n, float cap, hipStream_t s) {
+  if (n <= 0) return 0;
+  if (!(cap > 0.f)) return -1;
+  hipLaunchKernelGGL(tanh_cap_kernel, dim3(ew_grid(n)), dim3(256), 0, s, x, n, cap);
+  return (int)hipGetLastError();
 }
 
 extern "C" int mx_relu_sq(void* x, int bf16, long n, hipStream_t s) {

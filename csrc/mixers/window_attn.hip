@@ -4,11 +4,14 @@
 //
 // Query head a = h * maps + m (head h, map m) reads key head (h / rep) * maps + m and
 // value head h / rep, rep = heads / kv_heads.  Position i sees key j iff 0 <= i - j
-// (< window when window > 0).  score = q.k * scale - r1[a] ln(1 + r2[a] (i - j));
-// weight = softmax over the visible keys, or sigmoid(score + pb[a]) unnormalised.
+// (< window when window > 0).  s = q.k * scale, capped to softcap tanh(s / softcap) when
+// softcap > 0; score = s - r1[a] ln(1 + r2[a] (i - j)); weight = softmax over the visible
+// keys, or sigmoid(score + pb[a]) unnormalised.  A softmax may carry a sink: one more
+// term exp(sink) in its denominator, a key that is always visible and has no value.
 // Queries, scores, weights and sums are fp32; the caches hold fp32 or bf16 rows.
 //
 // Kernels: attn_prep (whole-projection RMS norms, rotary positions, cache writes),
+// conv_attn_prep (short causal convolution over time, per-head RMS norms, cache writes),
 // window_attn (one workgroup per (row, query head): decode rows and short segments),
 // band_weights (scores -> weights for the banded matrix products of long segments) and
 // diff_combine (two maps -> one gated, normed head output).
@@ -78,6 +81,77 @@ __global__ void attn_prep_kernel(float* __restrict__ q_out, const T* __restrict_
   }
   if (keep)
     for (int e = threadIdx.x; e < nv; e += NT) st(v_cache, slot * nv + e, ld(in, nq + nk + e));
+}
+
+// ---------------------------------------------------------------------------------
+// one workgroup per row of the fused [q | k | v] projection: a causal convolution over
+// time on every channel (taps along the row axis, the last tap on the row itself; rows
+// before the segment's first come from the state slot's history, zeros at position 0),
+// then an RMS norm of every head_dim chunk of q and k with one shared weight vector, fp32
+// throughout.  q leaves as fp32, k and v go to the row's cache slot.  The history is
+// updated afterwards by mx_conv_hist.
+// ---------------------------------------------------------------------------------
+template <typename T, typename TC, int NT>
+__global__ void conv_attn_prep_kernel(float* __restrict__ q_out, const T* __restrict__ qkv, long stride, int nq,
+                                      int nk, int nv, const float* __restrict__ conv_w, int taps,
+                                      const float* __restrict__ hist, const int* __restrict__ start,
+                                      const int* __restrict__ pos0, const int* __restrict__ slot, int num_segs,
+                                      int num_state_slots, const float* __restrict__ wq,
+                                      const float* __restrict__ wk, float eps, int head_dim,
+                                      const int* __restrict__ slots, TC* __restrict__ k_cache,
+                                      TC* __restrict__ v_cache, long num_slots) {
+  extern __shared__ float smem[];
+  const int channels = nq + nk + nv;
+  float* y = smem;                    // [channels]
+  float* rinv = smem + channels;      // [(nq + nk) / head_dim]
+  const int row = blockIdx.x;
+  if (row >= start[num_segs]) return;
+  int lo_s = 0, hi_s = num_segs;
+  while (hi_s - lo_s > 1) {
+    const int mid = (lo_s + hi_s) >> 1;
+    if (start[mid] <= row) lo_s = mid; else hi_s = mid;
+  }
+  const int s = lo_s;
+  const int r0 = start[s], rel = row - r0;
+  const int sl = slot[s];
+  const bool old = sl >= 0 && sl < num_state_slots && pos0[s] > 0;   // the slot's history counts
+  const float* h = hist + (long)(old ? sl : 0) * (taps - 1) * channels;
+  for (int c = threadIdx.x; c < channels; c += NT) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int src = rel - (taps - 1) + j;
+      float v;
+      if (src >= 0) v = ld(qkv, (long)(r0 + src) * stride + c);
+      else v = old ? h[(long)(taps - 1 + src) * channels + c] : 0.f;
+      acc += v * conv_w[(long)c * taps + j];
+    }
+    y[c] = acc;
+  }
+  __syncthreads();
+  const int chunks = (nq + nk) / head_dim;
+  const int lane = threadIdx.x & 63;
+  for (int ch = threadIdx.x >> 6; ch < chunks; ch += NT / 64) {
+    float ss = 0.f;
+    for (int i = lane; i < head_dim; i += 64) {
+      const float v = y[ch * head_dim + i];
+      ss += v * v;
+    }
+    ss = ft::wave_sum(ss);
+    if (lane == 0) rinv[ch] = 1.0f / sqrtf(ss / (float)head_dim + eps);
+  }
+  __syncthreads();
+  const long cs = slots[row];
+  const bool keep = cs >= 0 && cs < num_slots;
+  for (int e = threadIdx.x; e < nq + nk; e += NT) {
+    const bool is_q = e < nq;
+    const float* w = is_q ? wq : wk;
+    float v = y[e];
+    if (w != nullptr) v *= rinv[e / head_dim] * w[e % head_dim];
+    if (is_q) q_out[(long)row * nq + e] = v;
+    else if (keep) st(k_cache, cs * nk + (e - nq), v);
+  }
+  if (keep)
+    for (int e = threadIdx.x; e < nv; e += NT) st(v_cache, cs * nv + e, y[nq + nk + e]);
 }
 
 // ---------------------------------------------------------------------------------
@@ -161,7 +235,8 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
                    const int* __restrict__ kv_len, const int* __restrict__ bt, int bt_stride, int num_segs,
                    int heads, int maps, int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
                    const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ pb,
-                   int block_size, int num_blocks, int skip_from, int vec, int lpk) {
+                   int block_size, int num_blocks, int skip_from, int vec, int lpk, float softcap, int has_sink,
+                   float sink) {
   extern __shared__ float smem[];
   const int row = blockIdx.x, a = blockIdx.y;
   const int hq = heads * maps;
@@ -211,6 +286,7 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
       if (blk >= 0 && blk < num_blocks) {
         slot = blk * block_size + j % block_size;
         z = dot_row<TC>(k_cache + (long)slot * nk + (long)kh * dk, q_s, dk, vec != 0) * scale;
+        if (softcap > 0.f) z = softcap * tanhf(z / softcap);
         if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)(i - j));
       }
     }
@@ -284,10 +360,10 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
 #pragma unroll
       for (int w = 0; w < kWaves; ++w) acc += o_s[w * dv + c];
     } else {
-      float mm = -INFINITY;
+      float mm = has_sink ? sink : -INFINITY;
 #pragma unroll
       for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, ml_s[2 * w]);
-      float l = 0.f;
+      float l = has_sink ? expf(sink - mm) : 0.f;
 #pragma unroll
       for (int w = 0; w < kWaves; ++w) {
         const float f = ml_s[2 * w] == -INFINITY ? 0.f : expf(ml_s[2 * w] - mm);
@@ -308,7 +384,7 @@ template <int NT>
 __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, int first_pos, int key0,
                                     int heads, int maps, int kv_heads, int window, float scale, int sigmoid,
                                     const float* __restrict__ r1, const float* __restrict__ r2,
-                                    const float* __restrict__ pb) {
+                                    const float* __restrict__ pb, float softcap, int has_sink, float sink) {
   __shared__ float red[NT / 64];
   const int rep = heads / kv_heads;
   const int rr = blockIdx.x, gk = blockIdx.y;
@@ -323,6 +399,7 @@ __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, i
   const float c1 = r1 != nullptr ? r1[a] : 0.f, c2 = r1 != nullptr ? r2[a] : 0.f;
   auto score = [&](int c) {
     float z = sp[c] * scale;
+    if (softcap > 0.f) z = softcap * tanhf(z / softcap);
     if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)(i - key0 - c));
     return z;
   };
@@ -345,6 +422,7 @@ __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, i
   __syncthreads();
 #pragma unroll
   for (int w = 0; w < NT / 64; ++w) mx_ = fmaxf(mx_, red[w]);
+  if (has_sink) mx_ = fmaxf(mx_, sink);
   float sum = 0.f;
   for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) {
     const float p = expf(sp[c] - mx_);
@@ -352,6 +430,7 @@ __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, i
     sum += p;
   }
   sum = block_sum<NT>(sum, red);
+  if (has_sink) sum += expf(sink - mx_);
   const float inv = sum > 0.f ? 1.0f / sum : 0.f;
   for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) sp[c] *= inv;
 }
@@ -401,6 +480,35 @@ extern "C" int mx_attn_prep(float* q_out, const void* qkv, int bf16, long stride
   return (int)hipGetLastError();
 }
 
+extern "C" int mx_conv_hist(const void* x, int bf16, long x_stride, float* hist, const int* start, const int* pos0,
+                            const int* slot, int num_segs, int channels, int taps, int num_slots, hipStream_t s);
+
+extern "C" int mx_conv_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv,
+                                 const float* conv_w, int taps, float* hist, const int* start, const int* pos0,
+                                 const int* slot, int num_segs, int num_state_slots, const float* wq,
+                                 const float* wk, float eps, int head_dim, const int* slots, void* k_cache,
+                                 void* v_cache, int cache_bf16, long num_slots, long rows, hipStream_t s) {
+  if (rows <= 0 || num_segs <= 0) return 0;
+  if (head_dim < 1 || nq % head_dim || nk % head_dim || taps < 1 || nv < 0) return -1;
+  const int channels = nq + nk + nv;
+  const size_t shm = (size_t)(channels + (nq + nk) / head_dim) * sizeof(float);
+  if (shm > 64 * 1024) return -3;
+  const dim3 grid((unsigned)rows), block(256);
+#define MX_CPREP(T, TC)                                                                                       \
+  hipLaunchKernelGGL((conv_attn_prep_kernel<T, TC, 256>), grid, block, shm, s, q_out, (const T*)qkv, stride, nq, \
+                     nk, nv, conv_w, taps, hist, start, pos0, slot, num_segs, num_state_slots, wq, wk, eps,      \
+                     head_dim, slots, (TC*)k_cache, (TC*)v_cache, num_slots)
+  if (bf16 && cache_bf16) MX_CPREP(bf16_t, bf16_t);
+  else if (bf16) MX_CPREP(bf16_t, float);
+  else if (cache_bf16) MX_CPREP(float, bf16_t);
+  else MX_CPREP(float, float);
+#undef MX_CPREP
+  int rc = (int)hipGetLastError();
+  if (rc == 0 && taps > 1)
+    rc = mx_conv_hist(qkv, bf16, stride, hist, start, pos0, slot, num_segs, channels, taps, num_state_slots, s);
+  return rc;
+}
+
 extern "C" int mx_window_max_dv() { return 64 * kMaxVCols; }
 
 extern "C" int mx_window_attention(float* out, const float* q, const void* k_cache, const void* v_cache,
@@ -408,7 +516,8 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
                                    const int* bt, int bt_stride, int num_segs, long total_rows, int heads, int maps,
                                    int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
                                    const float* r1, const float* r2, const float* pb, int block_size,
-                                   int num_blocks, int skip_from, hipStream_t s) {
+                                   int num_blocks, int skip_from, float softcap, int has_sink, float sink,
+                                   hipStream_t s) {
   if (num_segs <= 0 || total_rows <= 0) return 0;
   if (dv < 1 || dv > mx_window_max_dv() || dk < 1 || heads % kv_heads || maps < 1) return -1;
   const int hq = heads * maps;
@@ -429,7 +538,8 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
   MX_DISPATCH_T(cache_bf16, hipLaunchKernelGGL((window_attn_kernel<T, V>), grid, block, shm, s, out, q,         \
                                                (const T*)k_cache, (const T*)v_cache, start, pos0, kv_len, bt,  \
                                                bt_stride, num_segs, heads, maps, kv_heads, dk, dv, window, scale, \
-                                               sigmoid, r1, r2, pb, block_size, num_blocks, skip_from, vec, lpk))
+                                               sigmoid, r1, r2, pb, block_size, num_blocks, skip_from, vec, lpk,  \
+                                               softcap, has_sink, sink))
   if (vecv) MX_WATTN(true);
   else MX_WATTN(false);
 #undef MX_WATTN
@@ -438,11 +548,13 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
 
 extern "C" int mx_band_weights(float* S, int gk, int rep_rows_total, int rows, int keys, int first_pos, int key0,
                                int heads, int maps, int kv_heads, int window, float scale, int sigmoid,
-                               const float* r1, const float* r2, const float* pb, hipStream_t s) {
+                               const float* r1, const float* r2, const float* pb, float softcap, int has_sink,
+                               float sink, hipStream_t s) {
   if (gk <= 0 || rep_rows_total <= 0 || keys <= 0) return 0;
   if (heads % kv_heads || gk != kv_heads * maps || rep_rows_total != heads / kv_heads * rows || gk > 65535) return -1;
   hipLaunchKernelGGL((band_weights_kernel<256>), dim3((unsigned)rep_rows_total, (unsigned)gk), dim3(256), 0, s, S,
-                     rows, keys, first_pos, key0, heads, maps, kv_heads, window, scale, sigmoid, r1, r2, pb);
+                     rows, keys, first_pos, key0, heads, maps, kv_heads, window, scale, sigmoid, r1, r2, pb, softcap,
+                     has_sink, sink);
   return (int)hipGetLastError();
 }
 
