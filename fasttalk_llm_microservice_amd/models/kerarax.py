@@ -231,13 +231,14 @@ PRESETS = {
         {"type": ATTENTION, "mixer": _att(3, 1, 8, 8, conv=2, softcap=10.0), "mlp": None},
         {"type": ATTENTION, "mixer": _att(4, 4, 16, 16, conv=4, softcap=10.0), "mlp": _moe(4, 1, 64, 0)},
     ]),
-    # a 2048-wide stack (benchmarks): 32 experts of ff 1408, top 4, and a shared expert of
-    # ff 2816 (about 50 M active weights per layer, as nulazen-2k)
+    # a 2048-wide stack (benchmarks): 32 experts, top 4, and a shared expert; two matrices per
+    # expert, sized so that a token's active expert weights equal those of nulazen-2k's
+    # three-matrix experts (38 M per layer)
     "kerarax-2k": _preset("kerarax-2k", 32768, 2048, [
-        {"type": ATTENTION, "mixer": _att(16, 4, 128, 128), "mlp": _moe(32, 4, 1408, 2816)} for _ in range(4)]),
-    # the same stack at 4096 width
+        {"type": ATTENTION, "mixer": _att(16, 4, 128, 128), "mlp": _moe(32, 4, 1536, 3072)} for _ in range(4)]),
+    # the same stack at 4096 width (64 experts, top 6, as nulazen-4k)
     "kerarax-4k": _preset("kerarax-4k", 32768, 4096, [
-        {"type": ATTENTION, "mixer": _att(32, 8, 128, 128), "mlp": _moe(32, 4, 2816, 5632)} for _ in range(4)]),
+        {"type": ATTENTION, "mixer": _att(32, 8, 128, 128), "mlp": _moe(64, 6, 2112, 4224)} for _ in range(4)]),
 }
 
 

@@ -69,7 +69,7 @@ def test_registry_and_config(tmp_path):
     assert architecture_of(resolve_model("bagasun-tiny")).name == "bagasun"
     assert architecture_of(resolve_model("tiny")).name == "llama"
     # the written configuration parses back to itself; an unknown mixer is refused
-    assert KX.config_from_dict(KX.config_to_dict(mc), "a") == mc
+    assert KX.config_from_dict(KX.config_to_dict(mc), mc.name) == mc
     bad = {**cfg, "layers": [{**cfg["layers"][0], "type": "mamba2"}]}
     with pytest.raises(ValueError):
         KX.config_from_dict(bad)
