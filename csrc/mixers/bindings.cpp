@@ -15,6 +15,9 @@ int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int r
 int mx_layer_norm(float* x, const void* y, int y_bf16, long y_stride, const float* w, const float* b, void* out,
                   void* cast, int out_bf16, int rows, int width, float eps, hipStream_t s);
 int mx_tanh_cap(float* x, long n, float cap, hipStream_t s);
+int mx_relu_sq_rows(void* out, const void* u, int bf16, long u_stride, long rows, int ff, hipStream_t s);
+int mx_gather_add_rows(float* out, const void* y, int y_bf16, const int* idx, const float* w, long rows, int top,
+                       int width, long y_rows, hipStream_t s);
 int mx_conv_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv,
                       const float* conv_w, int taps, float* hist, const int* start, const int* pos0, const int* slot,
                       int num_segs, int num_state_slots, const float* wq, const float* wk, float eps, int head_dim,
@@ -234,6 +237,25 @@ void head_rms_gate(Tensor out, Tensor o, Tensor w, Tensor gate, double eps, int6
 void relu_sq(Tensor x) {
   TORCH_CHECK(x.is_cuda() && is_act(x) && x.is_contiguous(), "x");
   chk(mx_relu_sq(x.data_ptr(), bf(x), x.numel(), stream()), "relu_sq");
+}
+
+void relu_sq_rows(Tensor out, Tensor u) {
+  check_rows(u, "u");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == u.scalar_type() && out.dim() == 2 &&
+              out.size(0) == u.size(0) && out.size(1) >= 1 && out.size(1) <= u.size(1), "out");
+  chk(mx_relu_sq_rows(out.data_ptr(), u.data_ptr(), bf(u), u.stride(0), u.size(0), (int)out.size(1), stream()),
+      "relu_sq_rows");
+}
+
+void gather_add_rows(Tensor out, Tensor y, Tensor idx, Tensor w) {
+  check_f32(out, "out");
+  check_i32(idx, "idx");
+  check_f32(w, "weights");
+  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && is_act(y) && y.dim() == 2 && out.dim() == 2 &&
+              y.size(1) == out.size(1) && idx.dim() == 2 && idx.size(0) == out.size(0) && w.sizes() == idx.sizes(),
+              "gather_add_rows shapes");
+  chk(mx_gather_add_rows(out.data_ptr<float>(), y.data_ptr(), bf(y), idx.data_ptr<int>(), w.data_ptr<float>(),
+                         out.size(0), (int)idx.size(1), (int)out.size(1), y.size(0), stream()), "gather_add_rows");
 }
 
 void clamp_swiglu(Tensor out, Tensor gu, double limit) {
@@ -624,6 +646,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_top_logits", &moe_top_logits);
   m.def("head_rms_gate", &head_rms_gate);
   m.def("relu_sq", &relu_sq);
+  m.def("relu_sq_rows", &relu_sq_rows);
+  m.def("gather_add_rows", &gather_add_rows);
   m.def("clamp_swiglu", &clamp_swiglu);
   m.def("side_gate", &side_gate);
   m.def("scale_add_rows", &scale_add_rows);

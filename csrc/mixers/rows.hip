@@ -142,6 +142,33 @@ __global__ void relu_sq_kernel(T* __restrict__ x, long n) {
   }
 }
 
+// out[r, c] = relu(u[r, c])^2 for the first ff columns of wider rows
+template <typename T>
+__global__ void relu_sq_rows_kernel(T* __restrict__ out, const T* __restrict__ u, long u_stride, long rows, int ff) {
+  const long n = rows * ff;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const float v = fmaxf(ld(u, (i / ff) * u_stride + i % ff), 0.f);
+    st(out, i, v * v);
+  }
+}
+
+// out[row] += sum_k w[row, k] * y[idx[row, k]]: combines the outputs of the experts each
+// row chose, y being in another row order (sorted by expert).  grid rows.
+template <typename TY>
+__global__ void gather_add_rows_kernel(float* __restrict__ out, const TY* __restrict__ y,
+                                       const int* __restrict__ idx, const float* __restrict__ w, int top,
+                                       int width, long y_rows) {
+  const long row = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const long src = idx[row * top + k];
+      if (src >= 0 && src < y_rows) acc += w[row * top + k] * ld(y, src * width + c);
+    }
+    out[row * width + c] += acc;
+  }
+}
+
 // rows [gate (ff) | up (ff) | ...]: g = min(gate, limit), u = clamp(up, +-limit),
 // out = g * sigmoid(1.702 g) * (u + 1)
 template <typename T>
@@ -289,6 +316,22 @@ extern "C" int mx_tanh_cap(float* x, long n, float cap, hipStream_t s) {
 extern "C" int mx_relu_sq(void* x, int bf16, long n, hipStream_t s) {
   if (n <= 0) return 0;
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((relu_sq_kernel<T>), dim3(ew_grid(n)), dim3(256), 0, s, (T*)x, n));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_relu_sq_rows(void* out, const void* u, int bf16, long u_stride, long rows, int ff, hipStream_t s) {
+  if (rows * ff <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((relu_sq_rows_kernel<T>), dim3(ew_grid(rows * ff)), dim3(256), 0, s,
+                                         (T*)out, (const T*)u, u_stride, rows, ff));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_gather_add_rows(float* out, const void* y, int y_bf16, const int* idx, const float* w, long rows,
+                                  int top, int width, long y_rows, hipStream_t s) {
+  if (rows <= 0 || top <= 0) return 0;
+  if (rows > 0x7fffffffL) return -1;
+  MX_DISPATCH_T(y_bf16, hipLaunchKernelGGL((gather_add_rows_kernel<T>), dim3((unsigned)rows), dim3(256), 0, s, out,
+                                           (const T*)y, idx, w, top, width, y_rows));
   return (int)hipGetLastError();
 }
 

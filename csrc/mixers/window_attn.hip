@@ -84,28 +84,32 @@ __global__ void attn_prep_kernel(float* __restrict__ q_out, const T* __restrict_
 }
 
 // ---------------------------------------------------------------------------------
-// one workgroup per row of the fused [q | k | v] projection: a causal convolution over
-// time on every channel (taps along the row axis, the last tap on the row itself; rows
-// before the segment's first come from the state slot's history, zeros at position 0),
-// then an RMS norm of every head_dim chunk of q and k with one shared weight vector, fp32
-// throughout.  q leaves as fp32, k and v go to the row's cache slot.  The history is
-// updated afterwards by mx_conv_hist.
+// one wave per (row, chunk) of the fused [q | k | v] projection, a chunk being one head
+// of q or k (head_dim channels) or up to head_dim channels of v: a causal convolution
+// over time on every channel (taps along the row axis, the last tap on the row itself;
+// rows before the segment's first come from the state slot's history, zeros at position
+// 0), then, for q and k, the head's RMS norm with one weight vector shared by the heads,
+// fp32 throughout.  The convolved chunk waits in the wave's LDS strip between the two
+// passes.  q leaves as fp32, k and v go to the row's cache slot.  The history is
+// updated afterwards by mx_conv_hist.  grid (rows, ceil(chunks / 4)), 4 waves.
 // ---------------------------------------------------------------------------------
-template <typename T, typename TC, int NT>
-__global__ void conv_attn_prep_kernel(float* __restrict__ q_out, const T* __restrict__ qkv, long stride, int nq,
-                                      int nk, int nv, const float* __restrict__ conv_w, int taps,
-                                      const float* __restrict__ hist, const int* __restrict__ start,
-                                      const int* __restrict__ pos0, const int* __restrict__ slot, int num_segs,
-                                      int num_state_slots, const float* __restrict__ wq,
-                                      const float* __restrict__ wk, float eps, int head_dim,
-                                      const int* __restrict__ slots, TC* __restrict__ k_cache,
-                                      TC* __restrict__ v_cache, long num_slots) {
+template <typename T, typename TC>
+__global__ void __launch_bounds__(256)
+conv_attn_prep_kernel(float* __restrict__ q_out, const T* __restrict__ qkv, long stride, int nq, int nk, int nv,
+                      const float* __restrict__ conv_w, int taps, const float* __restrict__ hist,
+                      const int* __restrict__ start, const int* __restrict__ pos0, const int* __restrict__ slot,
+                      int num_segs, int num_state_slots, const float* __restrict__ wq,
+                      const float* __restrict__ wk, float eps, int head_dim, const int* __restrict__ slots,
+                      TC* __restrict__ k_cache, TC* __restrict__ v_cache, long num_slots) {
   extern __shared__ float smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* y = smem + wave * head_dim;
   const int channels = nq + nk + nv;
-  float* y = smem;                    // [channels]
-  float* rinv = smem + channels;      // [(nq + nk) / head_dim]
+  const int qk_chunks = (nq + nk) / head_dim;
+  const int chunks = qk_chunks + (nv + head_dim - 1) / head_dim;
+  const int ch = blockIdx.y * 4 + wave;
   const int row = blockIdx.x;
-  if (row >= start[num_segs]) return;
+  if (ch >= chunks || row >= start[num_segs]) return;
   int lo_s = 0, hi_s = num_segs;
   while (hi_s - lo_s > 1) {
     const int mid = (lo_s + hi_s) >> 1;
@@ -116,7 +120,11 @@ __global__ void conv_attn_prep_kernel(float* __restrict__ q_out, const T* __rest
   const int sl = slot[s];
   const bool old = sl >= 0 && sl < num_state_slots && pos0[s] > 0;   // the slot's history counts
   const float* h = hist + (long)(old ? sl : 0) * (taps - 1) * channels;
-  for (int c = threadIdx.x; c < channels; c += NT) {
+  const int c0 = ch * head_dim;
+  const int len = min(head_dim, channels - c0);
+  float ss = 0.f;
+  for (int i = lane; i < len; i += 64) {
+    const int c = c0 + i;
     float acc = 0.f;
     for (int j = 0; j < taps; ++j) {
       const int src = rel - (taps - 1) + j;
@@ -125,33 +133,24 @@ __global__ void conv_attn_prep_kernel(float* __restrict__ q_out, const T* __rest
       else v = old ? h[(long)(taps - 1 + src) * channels + c] : 0.f;
       acc += v * conv_w[(long)c * taps + j];
     }
-    y[c] = acc;
+    y[i] = acc;                        // each lane re-reads only what it wrote itself
+    ss += acc * acc;
   }
-  __syncthreads();
-  const int chunks = (nq + nk) / head_dim;
-  const int lane = threadIdx.x & 63;
-  for (int ch = threadIdx.x >> 6; ch < chunks; ch += NT / 64) {
-    float ss = 0.f;
-    for (int i = lane; i < head_dim; i += 64) {
-      const float v = y[ch * head_dim + i];
-      ss += v * v;
-    }
-    ss = ft::wave_sum(ss);
-    if (lane == 0) rinv[ch] = 1.0f / sqrtf(ss / (float)head_dim + eps);
-  }
-  __syncthreads();
   const long cs = slots[row];
   const bool keep = cs >= 0 && cs < num_slots;
-  for (int e = threadIdx.x; e < nq + nk; e += NT) {
-    const bool is_q = e < nq;
+  if (ch < qk_chunks) {
+    const bool is_q = c0 < nq;
     const float* w = is_q ? wq : wk;
-    float v = y[e];
-    if (w != nullptr) v *= rinv[e / head_dim] * w[e % head_dim];
-    if (is_q) q_out[(long)row * nq + e] = v;
-    else if (keep) st(k_cache, cs * nk + (e - nq), v);
+    float r = 1.f;
+    if (w != nullptr) r = 1.0f / sqrtf(ft::wave_sum(ss) / (float)head_dim + eps);
+    for (int i = lane; i < len; i += 64) {
+      const float v = w != nullptr ? y[i] * r * w[i] : y[i];
+      if (is_q) q_out[(long)row * nq + c0 + i] = v;
+      else if (keep) st(k_cache, cs * nk + (c0 - nq) + i, v);
+    }
+  } else if (keep) {
+    for (int i = lane; i < len; i += 64) st(v_cache, cs * nv + (c0 - nq - nk) + i, y[i]);
   }
-  if (keep)
-    for (int e = threadIdx.x; e < nv; e += NT) st(v_cache, cs * nv + e, y[nq + nk + e]);
 }
 
 // ---------------------------------------------------------------------------------
@@ -491,12 +490,13 @@ extern "C" int mx_conv_attn_prep(float* q_out, const void* qkv, int bf16, long s
   if (rows <= 0 || num_segs <= 0) return 0;
   if (head_dim < 1 || nq % head_dim || nk % head_dim || taps < 1 || nv < 0) return -1;
   const int channels = nq + nk + nv;
-  const size_t shm = (size_t)(channels + (nq + nk) / head_dim) * sizeof(float);
-  if (shm > 64 * 1024) return -3;
-  const dim3 grid((unsigned)rows), block(256);
+  const size_t shm = (size_t)4 * head_dim * sizeof(float);
+  const int chunks = (nq + nk) / head_dim + (nv + head_dim - 1) / head_dim;
+  if (shm > 64 * 1024 || rows > 0x7fffffffL || (chunks + 3) / 4 > 65535) return -3;
+  const dim3 grid((unsigned)rows, (unsigned)((chunks + 3) / 4)), block(256);
 #define MX_CPREP(T, TC)                                                                                       \
-  hipLaunchKernelGGL((conv_attn_prep_kernel<T, TC, 256>), grid, block, shm, s, q_out, (const T*)qkv, stride, nq, \
-                     nk, nv, conv_w, taps, hist, start, pos0, slot, num_segs, num_state_slots, wq, wk, eps,      \
+  hipLaunchKernelGGL((conv_attn_prep_kernel<T, TC>), grid, block, shm, s, q_out, (const T*)qkv, stride, nq, nk, \
+                     nv, conv_w, taps, hist, start, pos0, slot, num_segs, num_state_slots, wq, wk, eps,         \
                      head_dim, slots, (TC*)k_cache, (TC*)v_cache, num_slots)
   if (bf16 && cache_bf16) MX_CPREP(bf16_t, bf16_t);
   else if (bf16) MX_CPREP(bf16_t, float);

@@ -572,6 +572,44 @@ def relu_sq(x):
     return ref.relu_sq(x)
 
 
+def relu_sq_rows(u, ff: int):
+    """relu(u[:, :ff])^2 of wider rows (a column range of a fused product), dense."""
+    if u.is_cuda:
+        out = torch.empty(u.shape[0], ff, dtype=u.dtype, device=u.device)
+        native_mixers().relu_sq_rows(out, u)
+        return out
+    return ref.relu_sq_rows(u, ff)
+
+
+def gather_add_rows(out, y, idx, w):
+    """out[r] (fp32, in place) += sum_k w[r, k] * y[idx[r, k]]; idx int32 [rows, top]."""
+    if out.is_cuda:
+        native_mixers().gather_add_rows(out, y, idx, w)
+    else:
+        ref.gather_add_rows(out, y, idx, w)
+
+
+def grouped_mm(a, w, offsets, counts=None):
+    """Rows of ``a`` [M, K] sorted by group; group g's rows (up to ``offsets[g]``, the
+    running sum of the group sizes, int32 on the device) times w[g]^T, w [G, N, K] ->
+    [M, N] in a's dtype.  bf16 on a GPU with K and N multiples of 8 is one grouped vendor
+    product (no host round trip); otherwise one product per group (``counts``: the group
+    sizes on the host, read from ``offsets`` when not given)."""
+    if a.is_cuda and a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and w.shape[1] % 8 == 0 \
+            and hasattr(torch, "_grouped_mm"):
+        return torch._grouped_mm(a, w.transpose(1, 2), offs=offsets)
+    if counts is None:
+        ends = offsets.tolist()
+        counts = [e - s for s, e in zip([0] + ends[:-1], ends)]
+    out = torch.empty(a.shape[0], w.shape[1], dtype=a.dtype, device=a.device)
+    s = 0
+    for g, n in enumerate(counts):
+        if n:
+            torch.mm(a[s:s + n], w[g].t(), out=out[s:s + n])
+        s += n
+    return out
+
+
 def side_gate(gpre, table, ids, col0: int, sd: int):
     """gelu_tanh(gpre) * table[ids, col0:col0+sd]."""
     if gpre.is_cuda:

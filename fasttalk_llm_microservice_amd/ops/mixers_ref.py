@@ -268,6 +268,15 @@ def relu_sq(x):
     return (r * r).to(x.dtype)
 
 
+def relu_sq_rows(u, ff):
+    r = torch.relu(u[:, :ff].float())
+    return (r * r).to(u.dtype)
+
+
+def gather_add_rows(out, y, idx, w):
+    out.add_((y.float()[idx.long()] * w.float()[:, :, None]).sum(1))
+
+
 def gelu_tanh(z):
     return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z * z * z)))
 

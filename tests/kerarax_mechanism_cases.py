@@ -110,7 +110,8 @@ def run(case, device, dtype):
     elif case == "layer_norm":
         for width in (24, 300):
             w, b = (1 + _rand(g, width, s=0.2)).to(device), _rand(g, width, s=0.2).to(device)
-            x0, y = _rand(g, 5, width) + 3.0, _rand(g, 5, width, s=4.0) - 2.0       # means far from 0
+            x0 = _rand(g, 5, width) + 3.0
+            y = (_rand(g, 5, width, s=4.0) - 2.0).bfloat16().float()                # means far from 0
             x = x0.clone().to(device)
             h = M.add_layer_norm_rows(x, y.to(device, dtype), w, b, EPS, dtype)
             want = x0 + O.layer_norm(y, w.cpu(), b.cpu(), EPS)
