@@ -15,6 +15,8 @@ int mx_embed_rows(float* out, const int* ids, const void* table, int bf16, int r
 int mx_layer_norm(float* x, const void* y, int y_bf16, long y_stride, const float* w, const float* b, void* out,
                   void* cast, int out_bf16, int rows, int width, float eps, hipStream_t s);
 int mx_tanh_cap(float* x, long n, float cap, hipStream_t s);
+int mx_grouped_gemm(void* C, const void* A, const void* W, const int* offs, int groups, long M, int N, int K,
+                    hipStream_t s);
 int mx_relu_sq_rows(void* out, const void* u, int bf16, long u_stride, long rows, int ff, hipStream_t s);
 int mx_gather_add_rows(float* out, const void* y, int y_bf16, const int* idx, const float* w, long rows, int top,
                        int width, long y_rows, hipStream_t s);
@@ -24,6 +26,8 @@ int mx_conv_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int 
                       const int* slots, void* k_cache, void* v_cache, int cache_bf16, long num_slots, long rows,
                       hipStream_t s);
 int mx_moe_top_logits(int* idx, float* wts, const float* z, long rows, int experts, int top, hipStream_t s);
+int mx_moe_route_top_logits(int* idx, float* wts, const void* h, int bf16, long h_stride, const float* router,
+                            const float* bias, long rows, int experts, int width, int top, hipStream_t s);
 int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, hipStream_t s);
 int mx_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv, const float* wq,
                  const float* wk, float eps, const float* table, int table_rows, int rot_dims, int head_dim,
@@ -258,6 +262,19 @@ void gather_add_rows(Tensor out, Tensor y, Tensor idx, Tensor w) {
                          out.size(0), (int)idx.size(1), (int)out.size(1), y.size(0), stream()), "gather_add_rows");
 }
 
+// out [M, N] = rows of a [M, K] (sorted by group, group g ends at offs[g]) times w[g]^T, w [G, N, K]; bf16
+void grouped_gemm(Tensor out, Tensor a, Tensor w, Tensor offs) {
+  check_i32(offs, "offsets");
+  TORCH_CHECK(a.is_cuda() && a.is_contiguous() && a.scalar_type() == at::kBFloat16 && a.dim() == 2, "a: bf16 [M, K]");
+  TORCH_CHECK(w.is_cuda() && w.is_contiguous() && w.scalar_type() == at::kBFloat16 && w.dim() == 3 &&
+              w.size(2) == a.size(1) && offs.numel() == w.size(0), "w: bf16 [G, N, K], offsets [G]");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == at::kBFloat16 && out.dim() == 2 &&
+              out.size(0) == a.size(0) && out.size(1) == w.size(1), "out: bf16 [M, N]");
+  TORCH_CHECK(a.size(1) % 8 == 0 && a.size(1) >= 8, "K must be a multiple of 8");
+  chk(mx_grouped_gemm(out.data_ptr(), a.data_ptr(), w.data_ptr(), offs.data_ptr<int>(), (int)w.size(0), a.size(0),
+                      (int)w.size(1), (int)a.size(1), stream()), "grouped_gemm");
+}
+
 void clamp_swiglu(Tensor out, Tensor gu, double limit) {
   check_rows(gu, "gu");
   const int64_t ff = gu.size(1) / 2;
@@ -444,6 +461,22 @@ void moe_top_logits(Tensor idx, Tensor wts, Tensor z, int64_t top) {
               wts.numel() == z.size(0) * top, "moe_top_logits shapes");
   chk(mx_moe_top_logits(idx.data_ptr<int>(), wts.data_ptr<float>(), z.data_ptr<float>(), z.size(0), (int)z.size(1),
                         (int)top, stream()), "moe_top_logits");
+}
+
+void moe_route_top_logits(Tensor idx, Tensor wts, Tensor h, Tensor router, OptT bias, int64_t top) {
+  check_i32(idx, "idx");
+  check_f32(wts, "wts");
+  check_rows(h, "h");
+  check_f32(router, "router");
+  TORCH_CHECK(router.dim() == 2 && router.size(1) == h.size(1) && top >= 1 && top <= router.size(0) &&
+              idx.numel() == h.size(0) * top && wts.numel() == h.size(0) * top, "moe_route_top_logits shapes");
+  if (bias) {
+    check_f32(*bias, "router bias");
+    TORCH_CHECK(bias->numel() == router.size(0), "router bias size");
+  }
+  chk(mx_moe_route_top_logits(idx.data_ptr<int>(), wts.data_ptr<float>(), h.data_ptr(), bf(h), h.stride(0),
+                              router.data_ptr<float>(), bias ? bias->data_ptr<float>() : nullptr, h.size(0),
+                              (int)router.size(0), (int)router.size(1), (int)top, stream()), "moe_route_top_logits");
 }
 
 // relu_sq: the experts' first matrix is [ff, width] (up alone) instead of [2 ff, width] (gate | up)
@@ -644,10 +677,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("tanh_cap", &tanh_cap);
   m.def("conv_attn_prep", &conv_attn_prep);
   m.def("moe_top_logits", &moe_top_logits);
+  m.def("moe_route_top_logits", &moe_route_top_logits);
   m.def("head_rms_gate", &head_rms_gate);
   m.def("relu_sq", &relu_sq);
   m.def("relu_sq_rows", &relu_sq_rows);
   m.def("gather_add_rows", &gather_add_rows);
+  m.def("grouped_gemm", &grouped_gemm);
   m.def("clamp_swiglu", &clamp_swiglu);
   m.def("side_gate", &side_gate);
   m.def("scale_add_rows", &scale_add_rows);

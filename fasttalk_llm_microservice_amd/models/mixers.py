@@ -434,6 +434,8 @@ class MoEFF:
         if self.routing == "grouped_softmax":
             z = F.linear(h.float(), self.router)
             return M.moe_topk(z, self.correction, self.top, self.groups, self.keep)
+        if h.shape[0] <= self.PAIR_ROWS:
+            return M.moe_route_top_logits(h, self.router, self.router_bias, self.top)
         return M.moe_top_logits(F.linear(h.float(), self.router, self.router_bias), self.top)
 
     def _act(self, u):
@@ -447,23 +449,23 @@ class MoEFF:
             # decode-size steps: per-pair weight streaming, nothing read back on the host
             M.moe_pairs(out, h, idx, wts, self.wgu, self.wdown, self.limit, self.act)
             return self._shared(out, h)
+        # rows sorted by expert: each expert's rows are one group of two grouped products
         flat = idx.view(-1).long()
         order = torch.argsort(flat, stable=True)
-        counts = torch.bincount(flat, minlength=self.e).tolist()
-        rows = (order // self.top).int()
-        w = wts.view(-1).index_select(0, order)
-        hs = h.index_select(0, rows.long())
-        a = 0
-        for e, n in enumerate(counts):
-            if n == 0:
-                continue
-            y = self._act(F.linear(hs[a:a + n], self.wgu[e]))
-            M.scale_add_rows(out, F.linear(y, self.wdown[e]), rows[a:a + n], w[a:a + n])
-            a += n
+        offs = torch.bincount(flat, minlength=self.e).cumsum(0).int()
+        hs = h.index_select(0, order // self.top)
+        # group sizes on the host only where a product runs group by group
+        counts = None if M.grouped_mm_is_one_product(hs, self.wgu) and self.wdown.shape[2] % 8 == 0 \
+            else torch.bincount(flat, minlength=self.e).tolist()   # K of both products a multiple of 8
+        y = self._act(M.grouped_mm(hs, self.wgu, offs, counts))
+        d = M.grouped_mm(y, self.wdown, offs, counts)
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(order.numel(), device=order.device)
+        M.gather_add_rows(out, d, inv.view(t, self.top).int(), wts)
         return self._shared(out, h)
 
     # rows up to which every (row, expert) pair streams its expert's weights (decode);
-    # above, rows are sorted by expert and each expert runs one tiled product
+    # above, rows are sorted by expert and run as grouped products
     PAIR_ROWS = 64
 
     def _shared(self, out, h):
@@ -473,7 +475,7 @@ class MoEFF:
             if self.act == "clamp_glu":
                 y = M.clamp_swiglu(u, self.shared_limit)
             else:
-                y = M.relu_sq(u[:, :-1].contiguous())
+                y = M.relu_sq_rows(u, u.shape[1] - 1)
             M.scale_add_rows(out, F.linear(y, wdown), None, u[:, -1].contiguous(), sigmoid=True)
         return out
 

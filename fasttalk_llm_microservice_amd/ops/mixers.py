@@ -535,6 +535,18 @@ def moe_top_logits(z, top: int):
     return ref.moe_top_logits(z, top)
 
 
+def moe_route_top_logits(h, router, bias, top: int):
+    """:func:`moe_top_logits` of z = router h + bias (fp32 router [E, width] and bias, h fp32
+    or bf16, fp32 accumulation) in one launch: the router of few rows (decode steps)."""
+    if h.is_cuda:
+        t = h.shape[0]
+        idx = torch.empty(t, top, dtype=torch.int32, device=h.device)
+        wts = torch.empty(t, top, dtype=torch.float32, device=h.device)
+        native_mixers().moe_route_top_logits(idx, wts, h, router, bias, top)
+        return idx, wts
+    return ref.moe_top_logits(torch.nn.functional.linear(h.float(), router, bias), top)
+
+
 def moe_pairs(out, h, idx, wts, wgu, wdown, limit: float = 0.0, act: str = "clamp_glu"):
     """Few rows (decode): out (fp32, in place) += sum_k wts[:, k] * expert_{idx[:, k]}(h),
     every (row, expert) pair streaming its expert's first matrix ([gate | up] with the
@@ -589,15 +601,21 @@ def gather_add_rows(out, y, idx, w):
         ref.gather_add_rows(out, y, idx, w)
 
 
+def grouped_mm_is_one_product(a, w) -> bool:
+    """Whether :func:`grouped_mm` runs as one kernel without reading group sizes on the host."""
+    return bool(a.is_cuda and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0)
+
+
 def grouped_mm(a, w, offsets, counts=None):
     """Rows of ``a`` [M, K] sorted by group; group g's rows (up to ``offsets[g]``, the
     running sum of the group sizes, int32 on the device) times w[g]^T, w [G, N, K] ->
-    [M, N] in a's dtype.  bf16 on a GPU with K and N multiples of 8 is one grouped vendor
-    product (no host round trip); otherwise one product per group (``counts``: the group
+    [M, N] in a's dtype.  bf16 on a GPU with K a multiple of 8 is one grouped MFMA kernel
+    (no host round trip); otherwise one vendor product per group (``counts``: the group
     sizes on the host, read from ``offsets`` when not given)."""
-    if a.is_cuda and a.dtype == torch.bfloat16 and a.shape[1] % 8 == 0 and w.shape[1] % 8 == 0 \
-            and hasattr(torch, "_grouped_mm"):
-        return torch._grouped_mm(a, w.transpose(1, 2), offs=offsets)
+    if grouped_mm_is_one_product(a, w):
+        out = torch.empty(a.shape[0], w.shape[1], dtype=a.dtype, device=a.device)
+        native_mixers().grouped_gemm(out, a.contiguous(), w, offsets)
+        return out
     if counts is None:
         ends = offsets.tolist()
         counts = [e - s for s, e in zip([0] + ends[:-1], ends)]

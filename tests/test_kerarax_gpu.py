@@ -182,3 +182,33 @@ def test_graph_replays_of_new_kernels():
         torch.testing.assert_close(x, want_x, rtol=1e-6, atol=1e-6)
         torch.testing.assert_close(hist, want_h, rtol=0, atol=0)
         _ = (torch.randn(64, 64, device="cuda") @ torch.randn(64, 64, device="cuda")).sum().item()
+
+
+@pytest.mark.parametrize("shape", [(70, 24, 20, 5), (333, 40, 100, 7), (1000, 256, 192, 16), (64, 64, 64, 1),
+                                   (2048, 512, 136, 32)])
+def test_grouped_product_kernel(shape):
+    """The grouped expert product against one product per group: empty groups, groups that
+    are no multiple of the row tile, N and K that are no multiples of the tile sizes."""
+    from fasttalk_llm_microservice_amd.ops import mixers as M
+
+    m, k, n, groups = shape
+    g = torch.Generator().manual_seed(m + k)
+    a = torch.randn(m, k, generator=g).to("cuda", torch.bfloat16)
+    w = (torch.randn(groups, n, k, generator=g) * k ** -0.5).to("cuda", torch.bfloat16)
+    flat = torch.randint(0, groups, (m,), generator=g)
+    if groups > 2:
+        flat[flat == 1] = 0                      # an empty group in the middle
+        flat[flat == groups - 1] = 0             # and at the end
+    counts = torch.bincount(flat, minlength=groups)
+    offs = counts.cumsum(0).int().cuda()
+    assert M.grouped_mm_is_one_product(a, w)
+    got = M.grouped_mm(a, w, offs)
+    want = torch.empty_like(got)
+    s = 0
+    for e, c in enumerate(counts.tolist()):
+        want[s:s + c] = (a[s:s + c].float() @ w[e].float().t()).to(torch.bfloat16)
+        s += c
+    torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2)
+    # fp32 rows take one product per group and give the same
+    got32 = M.grouped_mm(a.float(), w.float(), offs)
+    torch.testing.assert_close(got32, want.float(), rtol=1e-2, atol=1e-2)
