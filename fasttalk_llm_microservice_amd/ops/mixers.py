@@ -273,7 +273,7 @@ def mm_f32(a, b):
 
 
 # bytes of fp32 scores the product path holds at once
-PRODUCT_SCORE_BYTES = 256 << 20
+PRODUCT_SCORE_BYTES = 1 << 30
 
 
 def latent_attention_products(out, qa, qr, cache, seg: Segments, scale: float, rank: int,
@@ -462,7 +462,8 @@ def window_attention_products(out, q, k_cache, v_cache, seg: Segments, spec: Win
         n = b - a
         if n < min_rows:
             continue
-        step = PRODUCT_CHUNK_ROWS if sp.window <= 0 else max(PRODUCT_CHUNK_ROWS, min(sp.window, 1024))
+        # without a window a chunk sees every earlier key anyway: long chunks, few launches
+        step = PRODUCT_FULL_CHUNK_ROWS if sp.window <= 0 else max(PRODUCT_CHUNK_ROWS, min(sp.window, 1024))
         # the fp32 scores of a chunk ([heads*maps, rows, keys]) stay under PRODUCT_SCORE_BYTES
         span = sp.window if sp.window > 0 else kv_len[s]
         while step > 32 and 4 * sp.heads * sp.maps * step * (step + span) > PRODUCT_SCORE_BYTES:
@@ -493,6 +494,9 @@ def window_attention_products(out, q, k_cache, v_cache, seg: Segments, spec: Win
 # rows of a segment that one pair of banded products covers (at least; a window wider
 # than this takes a chunk of its own width, up to 1024 rows)
 PRODUCT_CHUNK_ROWS = 256
+# rows per chunk when every earlier key is visible (halved until the chunk's scores fit
+# PRODUCT_SCORE_BYTES)
+PRODUCT_FULL_CHUNK_ROWS = 2048
 
 
 def diff_combine(a, gate, lam: float, post_scale: float, eps: float, heads: int, dv: int, out_dtype):

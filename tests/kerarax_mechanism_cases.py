@@ -9,7 +9,7 @@ import kerarax_oracle as O
 from fasttalk_llm_microservice_amd.models import mixers as X
 from fasttalk_llm_microservice_amd.ops import mixers as M
 
-CASES = ["embedding", "layer_norm", "attention", "attention_products", "attention_one_tap_wide_value",
+CASES = ["embedding", "layer_norm", "attention", "attention_products", "attention_product_chunks", "attention_one_tap_wide_value",
          "attention_long_taps", "attention_far_key", "attention_sink", "attention_cap", "router", "experts_pairs",
          "experts_sorted", "experts_all_chosen_no_shared", "logit_cap"]
 EPS = 1e-5
@@ -126,6 +126,16 @@ def run(case, device, dtype):
     elif case == "attention_products":
         _attention(device, dtype, host=True, T=77, cuts=(None, 33, 40, 44))
         _attention(device, dtype, host=True, T=77, H=3, G=1, dk=16, dv=70, cuts=(None, 35))
+    elif case == "attention_product_chunks":
+        # a long segment is cut into chunks of rows; each sees the keys up to its own last row
+        old = M.PRODUCT_FULL_CHUNK_ROWS, M.PRODUCT_SCORE_BYTES
+        try:
+            M.PRODUCT_FULL_CHUNK_ROWS = 40
+            _attention(device, dtype, host=True, T=150, cuts=(None, 33, 100))
+            M.PRODUCT_SCORE_BYTES = 4 * 4 * 35 * 150      # the memory bound halves the chunks again
+            _attention(device, dtype, host=True, T=150, cuts=(None, 70))
+        finally:
+            M.PRODUCT_FULL_CHUNK_ROWS, M.PRODUCT_SCORE_BYTES = old
     elif case == "attention_one_tap_wide_value":
         _attention(device, dtype, host=False, H=2, G=2, dk=6, dv=72, taps=1)
     elif case == "attention_long_taps":
