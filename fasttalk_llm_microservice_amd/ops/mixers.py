@@ -1,9 +1,12 @@
 """Sequence-mixer and mixture-of-experts ops: latent (low-rank KV) attention over a
 paged latent cache, windowed attention (softmax or sigmoid weights, distance bias,
-several score maps per head) over a paged key / value cache, the gated delta-rule
-recurrence with per-channel decay and the selective state-space scan over state slots,
-short causal convolutions, grouped top-k routing, clamped-GLU experts, and the
-fp32-residual norms that tie them together.
+several score maps per head, capped scores, a sink in the softmax) over a paged key /
+value cache, the gated delta-rule recurrence with per-channel decay and the selective
+state-space scan over state slots, short causal convolutions (alone, or fused with
+per-head norms and the cache write), routing (grouped softmax top-k, or top-k on the
+logits), clamped-GLU and relu^2 experts (per-pair kernels for few rows, a grouped product
+for many), and the fp32-residual norms (RMS pre/post norms, layer norm with bias) that tie
+them together.
 
 GPU tensors run the gfx950 kernels of the ``_C_mixers`` extension (``csrc/mixers``),
 fp32 or bf16 activations with fp32 statistics / scores / state; CPU tensors run the
