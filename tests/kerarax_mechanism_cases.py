@@ -175,6 +175,13 @@ def run(case, device, dtype):
                 assert idx.cpu().long().tolist() == wi.tolist()
             torch.testing.assert_close(w.cpu(), ww, rtol=1e-5, atol=1e-6)
             assert torch.allclose(w.sum(-1).cpu(), torch.ones(9), atol=1e-5)
+        # logits formed by the router kernel itself (few rows): widths with and without 16-byte rows
+        for width in (64, 50, 7):
+            h, rw, rb = _rand(g, 9, width), _rand(g, 13, width, s=0.5), _rand(g, 13, s=0.5)
+            idx, w = M.moe_route_top_logits(h.to(device, dtype), rw.to(device), rb.to(device), 4)
+            wi, ww = O.route(h @ rw.T + rb, 4)
+            assert idx.cpu().long().tolist() == wi.tolist()
+            torch.testing.assert_close(w.cpu(), ww, rtol=1e-4, atol=1e-5)
     elif case == "experts_pairs":
         _moe(device, dtype, 9, 6, 2, 20, 12)
     elif case == "experts_sorted":
