@@ -170,7 +170,7 @@ class WindowedAttention:
     PRODUCT_ROWS = 32
 
     def __init__(self, spec: M.WindowSpec, wqkv: torch.Tensor, bias: Optional[torch.Tensor],
-                 wo: torch.Tensor, eps: float, dtype):
+                 wo: torch.Tensor, eps: float, dtype, cache_of: Optional[int] = None):
         sp = spec
         if sp.heads % sp.kv_heads:
             raise ValueError("heads must be a multiple of kv_heads")
@@ -178,14 +178,21 @@ class WindowedAttention:
         self.nq = sp.heads * sp.maps * sp.dk
         self.nk = sp.kv_heads * sp.maps * sp.dk
         self.nv = sp.kv_heads * sp.dv
-        if wqkv.shape[0] < self.nq + self.nk + self.nv or wo.shape[1] != sp.heads * sp.dv:
+        # a layer that reads another layer's keys and values (``cache_of``: that layer's
+        # index) projects queries only and owns no pages: the model body hands it the
+        # other layer's cache
+        self.cache_of = cache_of
+        need = self.nq if cache_of is not None else self.nq + self.nk + self.nv
+        if wqkv.shape[0] < need or wo.shape[1] != sp.heads * sp.dv:
             raise ValueError("attention projections do not fit the head sizes")
         self.wqkv, self.bias, self.wo = wqkv, bias, wo
 
     def cache_bytes_per_token(self, elem_bytes: int) -> int:
-        return (self.nk + self.nv) * elem_bytes
+        return 0 if self.cache_of is not None else (self.nk + self.nv) * elem_bytes
 
     def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        if self.cache_of is not None:
+            return None
         return (torch.zeros(num_blocks, block_size, self.nk, dtype=dtype, device=device),
                 torch.zeros(num_blocks, block_size, self.nv, dtype=dtype, device=device))
 
@@ -307,6 +314,141 @@ class ConvSinkAttention(WindowedAttention):
         return F.linear(o.view(h.shape[0], -1).to(self.dtype), self.wo)
 
 
+class BiasedWindowAttention(WindowedAttention):
+    """Grouped-query softmax attention without rotation.  All rows of q together (and all
+    rows of k together) pass one RMS norm with a weight per row; the score of query i and
+    key j gains rel[bucket(i - j), head] from a table of ``rel.shape[0]`` rows -- distances
+    below half the rows have a row each, larger ones share rows in logarithmic steps up to
+    ``bias_reach`` (:func:`ops.mixers.distance_bias_table`); a position sees the last
+    ``window`` positions and, whatever the window, the first ``keep_first`` of the
+    sequence.  The concatenated heads are multiplied by sigmoid(W_g h) before the output
+    projection.  With ``cache_of`` the layer has no k / v projections of its own and
+    attends to the pages of the layer it names (keys as cached there, after that layer's
+    norm)."""
+
+    def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
+                 keep_first: int, scale: float, bias_reach: int, eps: float, dtype, device,
+                 cache_of: Optional[int] = None):
+        f32 = lambda n: get(n).to(device, torch.float32).contiguous()   # noqa: E731
+        rel = f32("rel")
+        if rel.dim() != 2 or rel.shape[1] != heads:
+            raise ValueError("distance bias table does not fit the heads")
+        spec = M.WindowSpec(heads, kv_heads, dim, vdim, int(window), float(scale), maps=1,
+                            keep_first=int(keep_first), dist_bias=M.distance_bias_table(rel, int(bias_reach)))
+        parts = [get("q")] + ([] if cache_of is not None else [get("k"), get("v")]) + [get("g")]
+        wqkv = torch.cat(parts, 0).to(device, dtype).contiguous()
+        super().__init__(spec, wqkv, None, get("o").to(device, dtype).contiguous(), eps, dtype, cache_of)
+        self.q_norm = f32("q.norm")
+        self.k_norm = None if cache_of is not None else f32("k.norm")
+        self.ng = heads * vdim
+        own = 0 if cache_of is not None else self.nk + self.nv
+        if wqkv.shape != (self.nq + own + self.ng, width) or self.q_norm.numel() != self.nq or \
+                (self.k_norm is not None and self.k_norm.numel() != self.nk):
+            raise ValueError("attention projections or norms do not fit the head sizes")
+        self.n_in = self.nq + own
+
+    def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
+        p = F.linear(h, self.wqkv)
+        if self.cache_of is not None:
+            q = M.attn_prep(p[:, :self.nq], self.nq, 0, self.q_norm, None, self.eps, None, 0, self.spec.dk,
+                            ctx.positions, ctx.slot_mapping, None, None)
+        else:
+            q = M.attn_prep(p[:, :self.n_in], self.nq, self.nk, self.q_norm, self.k_norm, self.eps, None, 0,
+                            self.spec.dk, ctx.positions, ctx.slot_mapping, cache[0], cache[1])
+        o = self.attend(q, ctx, cache)
+        return F.linear(M.sigmoid_gate(o.view(h.shape[0], -1), p[:, self.n_in:], self.dtype), self.wo)
+
+
+class RotaryBlockAttention(WindowedAttention):
+    """Grouped-query softmax attention with rotary positions on the first ``rot_dims``
+    entries of every head (entry i paired with i + rot_dims/2; frequencies optionally
+    ramped down for long contexts, ``rot_ramp`` = (factor, original, fast, slow) of
+    :func:`ops.mixers.ramp_frequencies`).  The sequence is cut into blocks of ``window``
+    positions counted from position 0, and a position sees the earlier positions of its
+    own block only (``window`` 0: every earlier position)."""
+
+    def __init__(self, get: Get, width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
+                 scale: float, rot_dims: int, rot_base: float, rot_ramp, eps: float, dtype, device, max_pos: int):
+        spec = M.WindowSpec(heads, kv_heads, dim, vdim, int(window), float(scale), maps=1, blocks=True)
+        wqkv = torch.cat([get("q"), get("k"), get("v")], 0).to(device, dtype).contiguous()
+        super().__init__(spec, wqkv, None, get("o").to(device, dtype).contiguous(), eps, dtype)
+        if rot_dims % 2 or rot_dims > dim or wqkv.shape != (self.nq + self.nk + self.nv, width):
+            raise ValueError("attention sizes do not fit")
+        self.rot_dims = int(rot_dims)
+        self.table = M.rope_table(max_pos, rot_dims, rot_base, device=device, ramp=rot_ramp) if rot_dims else None
+
+    def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
+        qkv = F.linear(h, self.wqkv)
+        q = M.attn_prep(qkv, self.nq, self.nk, None, None, self.eps, self.table, self.rot_dims, self.spec.dk,
+                        ctx.positions, ctx.slot_mapping, cache[0], cache[1])
+        o = self.attend(q, ctx, cache)
+        return F.linear(o.view(h.shape[0], -1).to(self.dtype), self.wo)
+
+
+class GatedLinearAttention:
+    """Linear attention with a decay per head and key channel: S <- diag(alpha) S + k v^T,
+    o = S^T q with q = W_q h dk^-1/2, alpha = sigmoid(W_a2 W_a1 h + b)^(1/tau).  Each head's
+    o is divided by its root mean square and multiplied by one weight vector shared by the
+    heads, the concatenated heads by silu(W_g h), then the output projection.  The state
+    [heads, dk, dv] is fp32 and lives in the sequence's state slot."""
+
+    def __init__(self, get: Get, width: int, heads: int, dim: int, vdim: int, tau: float, eps: float,
+                 dtype, device):
+        self.heads, self.dk, self.dv, self.tau, self.eps, self.dtype = heads, dim, vdim, float(tau), eps, dtype
+        a1 = get("a1")
+        self.nqkv = heads * (2 * dim + vdim)
+        self.ng = heads * vdim
+        # q | k | v | output gate | the decay's low-rank down-projection in one product
+        self.win = torch.cat([get("q"), get("k"), get("v"), get("g"), a1], 0).to(device, dtype).contiguous()
+        self.wa2 = get("a2").to(device, dtype).contiguous()
+        self.a_bias = get("a2.b").to(device, torch.float32).contiguous()
+        self.norm = get("norm").to(device, torch.float32).contiguous()
+        self.wo = get("o").to(device, dtype).contiguous()
+        if self.win.shape != (self.nqkv + self.ng + a1.shape[0], width) or \
+                self.wa2.shape != (heads * dim, a1.shape[0]) or self.a_bias.numel() != heads * dim or \
+                self.norm.numel() != vdim or self.wo.shape[1] != self.ng:
+            raise ValueError("linear-attention projections do not fit the head sizes")
+
+    def cache_bytes_per_token(self, elem_bytes: int) -> int:
+        return 0
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        return _state_slots(((self.heads, self.dk, self.dv),), num_slots, device)[0]
+
+    def __call__(self, h, ctx: StepContext, state) -> torch.Tensor:
+        p = F.linear(h, self.win)
+        a = F.linear(p[:, self.nqkv + self.ng:], self.wa2)
+        o = M.gated_linear_attention(p, a, self.a_bias, self.tau, state, ctx.seg, self.heads, self.dk, self.dv)
+        y = M.head_rms_gate(o, self.norm, p[:, self.nqkv:self.nqkv + self.ng], self.eps, self.heads, self.dv,
+                            self.dtype, silu=True)
+        return F.linear(y, self.wo)
+
+
+class SideBySide:
+    """Two mixers that read the same input; each output is divided by its root mean
+    square over the model width and multiplied by a weight vector of its own, and the
+    result is ``scale`` (one half) times their sum, in fp32.  The cache is the pair of the
+    two mixers' caches."""
+
+    def __init__(self, left, right, w_left: torch.Tensor, w_right: torch.Tensor, eps: float, device,
+                 scale: float = 0.5):
+        self.left, self.right, self.eps, self.scale = left, right, eps, float(scale)
+        self.w_left = w_left.to(device, torch.float32).contiguous()
+        self.w_right = w_right.to(device, torch.float32).contiguous()
+
+    def cache_bytes_per_token(self, elem_bytes: int) -> int:
+        return self.left.cache_bytes_per_token(elem_bytes) + self.right.cache_bytes_per_token(elem_bytes)
+
+    def alloc_cache(self, num_blocks, block_size, dtype, num_slots, device):
+        return (self.left.alloc_cache(num_blocks, block_size, dtype, num_slots, device),
+                self.right.alloc_cache(num_blocks, block_size, dtype, num_slots, device))
+
+    def __call__(self, h, ctx: StepContext, cache) -> torch.Tensor:
+        a = self.left(h, ctx, cache[0])
+        b = self.right(h, ctx, cache[1])
+        return M.dual_rms_mean(a, b, self.w_left, self.w_right, self.eps, self.scale)
+
+
 class StateSpaceMixer:
     """Selective state-space mixer with a scalar decay per head (state-space duality
     form): one input projection [z | x | B | C | dt], a short causal convolution with
@@ -354,13 +496,16 @@ class StateSpaceMixer:
 
 
 class GatedFF:
-    """down(gelu_tanh(gate h) * (up h))."""
+    """down(act(gate h) * (up h)), act = gelu_tanh or relu."""
 
-    def __init__(self, get: Get, dtype, device):
+    def __init__(self, get: Get, dtype, device, act: str = "gelu_tanh"):
+        if act not in ("gelu_tanh", "relu"):
+            raise ValueError("unknown feed-forward activation")
         self.wgu, self.down = _glu_weights(get, "", dtype, device)
+        self.glu = M.gelu_glu if act == "gelu_tanh" else M.relu_glu
 
     def __call__(self, h, ctx=None) -> torch.Tensor:
-        return F.linear(M.gelu_glu(F.linear(h, self.wgu)), self.down)
+        return F.linear(self.glu(F.linear(h, self.wgu)), self.down)
 
 
 class DenseFF:

@@ -43,7 +43,7 @@ def _ensure_loaded():
     if _loaded:
         return
     _loaded = True
-    from . import bagasun, kerarax, llama_arch, nulazen  # noqa: F401  (each registers itself)
+    from . import bagasun, fufipel, kerarax, llama_arch, nulazen  # noqa: F401  (each registers itself)
 
 
 def architecture_of(cfg) -> Architecture:

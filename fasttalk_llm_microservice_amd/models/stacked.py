@@ -17,6 +17,15 @@ read x itself, and a layer norm with weight and bias sits on each sublayer's out
 x += ln1(mixer(x)); x += ln2(ff(x)); the embedding rows (plus, optionally, a sinusoidal
 position vector) pass a layer norm before the first layer, and the final norm is a layer
 norm too.
+
+A model with ``norm_style = "shared_pre"`` has one RMS norm per layer that both sublayers
+read, and their outputs are added together: h = norm1(x); x += residual_mult *
+(mixer(h) + ff(h)).  The add and the next layer's norm are one kernel.
+
+Embedding extras: a pair table (``pair_embed``: a row chosen by a hash of the previous and
+the current token is added to the embedding row; the previous token of a sequence is kept
+in its state slot) and a scale on the logits; a model without a ``head`` tensor uses its
+embedding table as the head.
 """
 from __future__ import annotations
 
@@ -51,12 +60,24 @@ class StackedCache:
     """Per layer run, what its mixer's ``alloc_cache`` returned: paged tensors
     [num_blocks, block_size, ...] and / or per-slot state tensors [slots, ...]."""
 
-    def __init__(self, per_run: list):
+    def __init__(self, per_run: list, extra: Optional[dict] = None):
         self.per_run = per_run
+        self.extra = extra or {}      # state that belongs to no layer (per-slot tensors)
 
     def tensors(self):
-        for c in self.per_run:
-            yield from ((c,) if isinstance(c, torch.Tensor) else c)
+        seen = set()
+
+        def walk(c):
+            if isinstance(c, torch.Tensor):
+                if id(c) not in seen:      # a run that reads another run's pages holds the same tensors
+                    seen.add(id(c))
+                    yield c
+            elif c is not None:
+                for e in c:
+                    yield from walk(e)
+
+        yield from walk(self.per_run)
+        yield from walk(list(self.extra.values()))
 
 
 class StackedModel:
@@ -82,6 +103,9 @@ class StackedModel:
         self.embed_norm = None                  # (weight, bias) of the layer norm after the embedding
         self.final_bias = None
         self.logit_softcap = 0.0
+        self.logit_scale = 1.0
+        self.residual_mult = 1.0                # shared_pre: x += residual_mult * (mixer + ff)
+        self.pair_embed = None                  # (table, mul_prev, mul_cur, buckets)
         self.vocab_pad = 0
         self.mark_at = None
         self.layer_tap: Optional[list] = None   # tests: fp32 residual after every layer run
@@ -99,16 +123,19 @@ class StackedModel:
     def random_tensors(self, seed: int, device):
         raise NotImplementedError
 
-    def load_head(self, get):
-        """embed and head (rows padded to a multiple of 8) from the checkpoint."""
+    def load_head(self, get, has=lambda n: True):
+        """embed and head (rows padded to a multiple of 8) from the checkpoint; without a
+        ``head`` tensor the embedding table is the head."""
         dev, dt = self.device, self.dtype
         self.embed = get("embed").to(dev, dt).contiguous()
-        head = get("head").to(dev, dt)
+        head = (get("head") if has("head") else get("embed")).to(dev, dt)
         # the sampler reads logits rows in groups of 8: zero rows pad the head, and their
         # logits are set to -inf (never sampled; callers that want logits cut them off)
         self.vocab_pad = (-head.shape[0]) % 8
         if self.vocab_pad:
             head = torch.cat([head, torch.zeros(self.vocab_pad, head.shape[1], dtype=dt, device=dev)], 0)
+        elif not has("head"):
+            head = self.embed                    # one table for both
         self.head = head.contiguous()
 
     def norm_weight(self, t: torch.Tensor) -> torch.Tensor:
@@ -126,7 +153,7 @@ class StackedModel:
     def init_random(self, seed: int = 0, **_):
         on = self.device if self.device.type == "cuda" else "cpu"
         t = self.random_tensors(seed, on)
-        return self.load_tensors(t.__getitem__)
+        return self.load_tensors(t.__getitem__, t.__contains__)
 
     def resident_weight_bytes(self) -> int:
         seen, total = set(), 0
@@ -159,8 +186,18 @@ class StackedModel:
         dt = dtype or self.dtype
         if dt not in (torch.float32, torch.bfloat16):
             raise ValueError("paged caches are kept in the compute dtype")
-        return StackedCache([self.layers[i].mixer.alloc_cache(num_blocks, block_size, dt, num_slots, self.device)
-                             for i, _ in self.runs])
+        per_run = [self.layers[i].mixer.alloc_cache(num_blocks, block_size, dt, num_slots, self.device)
+                   for i, _ in self.runs]
+        # a mixer that reads another layer's keys and values gets that layer's (first) run's pages
+        for r, (i, _) in enumerate(self.runs):
+            src = getattr(self.layers[i].mixer, "cache_of", None)
+            if src is not None:
+                owner = next(q for q, (j, _) in enumerate(self.runs) if j == src)
+                per_run[r] = per_run[owner]
+        extra = {}
+        if self.pair_embed is not None:
+            extra["last_token"] = torch.full((max(num_slots, 1),), -1, dtype=torch.int32, device=self.device)
+        return StackedCache(per_run, extra)
 
     # ------------------------------------------------------------------ forward
     def forward(self, input_ids: torch.Tensor, meta, caches: StackedCache) -> torch.Tensor:
@@ -172,6 +209,8 @@ class StackedModel:
         ctx = StepContext(input_ids, meta.positions, meta.slot_mapping, seg)
         if self.norm_style == "layer_post":
             return self._forward_layer_post(input_ids, meta, ctx, caches)
+        if self.norm_style == "shared_pre":
+            return self._forward_shared_pre(input_ids, meta, ctx, caches)
         x = M.embed_rows(input_ids, self.embed, self.embed_scale)
         tap = self.layer_tap
         fuse_step = tap is None
@@ -233,10 +272,40 @@ class StackedModel:
             return rows.to(dt)
         return M.layer_norm_rows(rows, self.final_norm, self.final_bias, eps, dt)
 
+    def _forward_shared_pre(self, input_ids, meta, ctx, caches: StackedCache) -> torch.Tensor:
+        dt, eps, mult = self.dtype, self.cfg.rms_norm_eps, self.residual_mult
+        if self.pair_embed is not None:
+            table, mul_prev, mul_cur, buckets = self.pair_embed
+            x = M.pair_embed_rows(input_ids, self.embed, self.embed_scale, table, mul_prev, mul_cur, buckets, ctx.seg,
+                                  caches.extra["last_token"])
+        else:
+            x = M.embed_rows(input_ids, self.embed, self.embed_scale)
+        tap, mark = self.layer_tap, self.mark_at
+        nruns = len(self.runs)
+        h = M.add_scaled_rms_norm_rows(x, None, None, mult, self.layers[self.runs[0][0]].norm1, eps, dt) \
+            if nruns else None
+        for r, (li, _) in enumerate(self.runs):
+            if mark is not None and r == mark[0]:
+                mark[1].record()
+            L = self.layers[li]
+            y = L.mixer(h, ctx, caches.per_run[r])
+            f = L.ff(h, ctx) if L.ff is not None else None
+            nw = self.layers[self.runs[r + 1][0]].norm1 if r + 1 < nruns else None
+            h = M.add_scaled_rms_norm_rows(x, y, f, mult, nw, eps, dt)
+            if tap is not None:
+                tap.append(x.clone())
+        idx = meta.logits_indices
+        rows = x.index_select(0, idx) if idx.numel() != x.shape[0] else x
+        if rows.shape[0] == 0:
+            return rows.to(dt)
+        return M.rms_norm_rows(rows, self.final_norm, eps, dt)
+
     def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
         """fp32 logits [rows, vocab rounded up to a multiple of 8]; columns past the
         vocabulary are -inf.  With ``logit_softcap`` c > 0 the logits are c tanh(z / c)."""
         logits = self._head_product(h)
+        if self.logit_scale != 1.0:
+            logits *= self.logit_scale
         if self.logit_softcap:
             M.tanh_cap_(logits, self.logit_softcap)
         if self.vocab_pad:

@@ -147,11 +147,73 @@ def add_rms_norm_rows(residual: torch.Tensor, y: torch.Tensor, wb: torch.Tensor,
     return ref.add_rms_norm_rows(residual, y, wb, eps, add_vec, next_w, out_dtype, want_cast)
 
 
+def add_scaled_rms_norm_rows(residual: torch.Tensor, y1: Optional[torch.Tensor], y2: Optional[torch.Tensor],
+                             mult: float, next_w: Optional[torch.Tensor], eps: float, out_dtype):
+    """residual (fp32, in place) += mult * (y1 + y2); returns rms_norm(residual) * next_w in
+    ``out_dtype`` (None without ``next_w``).  y1 and y2 may be fp32 or bf16 each; y2, or
+    both, may be absent (then only the norm is taken).  The step between the layers of a
+    stack whose mixer and feed-forward read one shared norm and are added together."""
+    if residual.is_cuda:
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device) if next_w is not None else None
+        native_mixers().add_scaled_rms_norm(residual, y1, y2, float(mult), next_w, out, eps)
+        return out
+    return ref.add_scaled_rms_norm_rows(residual, y1, y2, mult, next_w, eps, out_dtype)
+
+
+def dual_rms_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float,
+                  scale: float = 0.5) -> torch.Tensor:
+    """fp32 scale * (rms_norm(a) * wa + rms_norm(b) * wb) of two rows of equal width: the
+    outputs of two mixers that run side by side, each normed on its own."""
+    if a.is_cuda:
+        out = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+        native_mixers().dual_rms_mean(out, a, b, wa, wb, eps, float(scale))
+        return out
+    return ref.dual_rms_mean(a, b, wa, wb, eps, scale)
+
+
+def pair_embed_add(x: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, mul_prev: int, mul_cur: int,
+                   buckets: int, seg: "Segments", last_tok: torch.Tensor) -> torch.Tensor:
+    """x (fp32 rows, in place) += table[(prev * mul_prev + cur * mul_cur) mod buckets], prev
+    being the token before the row's own in its sequence; a sequence's first token takes
+    row ``buckets``.  The token before a segment's first row comes from ``last_tok``
+    [slots] int32 (the sequence's state slot), which is then set to the segment's last
+    token."""
+    if x.is_cuda:
+        native_mixers().pair_embed_add(x, ids, table, int(mul_prev), int(mul_cur), int(buckets), seg.start,
+                                       seg.pos0, seg.slot, seg.num, last_tok, None, 1.0)
+        return x
+    return ref.pair_embed_add(x, ids, table, mul_prev, mul_cur, buckets, seg, last_tok)
+
+
+def pair_embed_rows(ids: torch.Tensor, embed: torch.Tensor, scale: float, table: torch.Tensor, mul_prev: int,
+                    mul_cur: int, buckets: int, seg: "Segments", last_tok: torch.Tensor) -> torch.Tensor:
+    """:func:`embed_rows` and :func:`pair_embed_add` in one launch: fp32 rows
+    embed[ids] * scale + table[hash(previous token, token)]."""
+    if ids.is_cuda:
+        x = torch.empty(ids.shape[0], embed.shape[1], dtype=torch.float32, device=ids.device)
+        native_mixers().pair_embed_add(x, ids, table, int(mul_prev), int(mul_cur), int(buckets), seg.start,
+                                       seg.pos0, seg.slot, seg.num, last_tok, embed, float(scale))
+        return x
+    return ref.pair_embed_add(ref.embed_rows(ids, embed, scale), ids, table, mul_prev, mul_cur, buckets, seg, last_tok)
+
+
+def sigmoid_gate(o: torch.Tensor, g: torch.Tensor, out_dtype) -> torch.Tensor:
+    """o * sigmoid(g) element by element (o fp32 [T, n]; g [T, n], may be a column range of
+    wider rows), rounded to ``out_dtype``."""
+    if o.is_cuda:
+        out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+        native_mixers().sigmoid_gate(out, o, g)
+        return out
+    return ref.sigmoid_gate(o, g, out_dtype)
+
+
 # ---------------------------------------------------------------------------------
 # rotary positions (partial, rotate-half pairs, fp32 angles)
 # ---------------------------------------------------------------------------------
 
 rope_table = ref.rope_table
+ramp_frequencies = ref.ramp_frequencies
+distance_bias_table = ref.distance_bias_table
 
 
 # ---------------------------------------------------------------------------------
@@ -190,13 +252,31 @@ def gated_delta_rule(qkv, a, b, a_log, dt_bias, state, seg: Segments, heads: int
     return ref.gated_delta_rule(qkv, a, b, a_log, dt_bias, state, seg, heads, kv_heads, dk, dv)
 
 
-def head_rms_gate(o, w, gate_pre, eps: float, heads: int, dv: int, out_dtype):
-    """Per head: o / rms(o) * w * sigmoid(gate_pre), rounded to ``out_dtype``."""
+def gated_linear_attention(qkv, a, a_bias, tau: float, state, seg: Segments, heads: int, dk: int,
+                           dv: int) -> torch.Tensor:
+    """Linear attention with a decay per head and key channel.
+
+    Rows of ``qkv`` are [q (heads*dk) | k (heads*dk) | v (heads*dv) | ...]; q is scaled by
+    dk^-1/2; decay = sigmoid(a + a_bias)^(1/tau), evaluated as exp(log sigmoid(.) / tau) in
+    fp32.  Per head and row:  S <- diag(decay) S + k v^T;  o = S^T q.  ``state`` [slots,
+    heads, dk, dv] fp32 is read (zeros at position 0) and left at the segment's last row.
+    Returns o fp32 [T, heads*dv]."""
+    if qkv.is_cuda:
+        o = torch.empty(qkv.shape[0], heads * dv, dtype=torch.float32, device=qkv.device)
+        native_mixers().gated_linear_attention(o, qkv, a, a_bias, float(tau), state, seg.start, seg.pos0,
+                                               seg.slot, seg.num, seg.max_rows, heads, dk, dv)
+        return o
+    return ref.gated_linear_attention(qkv, a, a_bias, tau, state, seg, heads, dk, dv)
+
+
+def head_rms_gate(o, w, gate_pre, eps: float, heads: int, dv: int, out_dtype, silu: bool = False):
+    """Per head: o / rms(o) * w * sigmoid(gate_pre) (or * silu(gate_pre)), rounded to
+    ``out_dtype``; ``gate_pre`` [T, heads*dv] may be a column range of wider rows."""
     if o.is_cuda:
         out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
-        native_mixers().head_rms_gate(out, o, w, gate_pre, eps, heads, dv)
+        native_mixers().head_rms_gate(out, o, w, gate_pre, eps, heads, dv, bool(silu))
         return out
-    return ref.head_rms_gate(o, w, gate_pre, eps, heads, dv, out_dtype)
+    return ref.head_rms_gate(o, w, gate_pre, eps, heads, dv, out_dtype, silu)
 
 
 # ---------------------------------------------------------------------------------
@@ -350,7 +430,8 @@ def attn_prep(qkv, nq: int, nk: int, q_norm_w, k_norm_w, eps: float, table, rot_
     values go to the rows' cache slots.  Optional steps, in this order: RMS norm of the
     whole q part and of the whole k part with weights ``q_norm_w`` / ``k_norm_w``; rotary
     positions on the first ``rot_dims`` entries of every ``head_dim`` chunk of q and k
-    (entry i paired with i + rot_dims/2, ``table`` = :func:`rope_table`)."""
+    (entry i paired with i + rot_dims/2, ``table`` = :func:`rope_table`).  Without caches
+    (``nk`` 0, rows of q alone) only the queries are prepared."""
     if qkv.is_cuda:
         q = torch.empty(qkv.shape[0], nq, dtype=torch.float32, device=qkv.device)
         native_mixers().attn_prep(q, qkv, nq, nk, q_norm_w, k_norm_w, eps, table, rot_dims, head_dim,
@@ -384,11 +465,14 @@ class WindowSpec:
     """A windowed attention's constants.  Query head a = h * maps + m (head h, score map
     m) reads key head floor(h / (heads / kv_heads)) * maps + m and value head
     floor(h / (heads / kv_heads)).  Position i sees j iff 0 <= i - j < window (window 0:
-    every earlier key).  s = q.k * scale; with ``softcap`` c > 0, s <- c tanh(s / c);
-    score = s - r1[a] ln(1 + r2[a] (i - j)); weight = softmax over the visible keys, or
-    sigmoid(score + pb[a]) without normalisation.  ``sink`` (a score, softmax only): the
-    softmax's denominator gains exp(sink), as if one more key with that score and no
-    value were always visible."""
+    every earlier key); with ``blocks`` the window is a block instead, j <= i and
+    floor(i / window) = floor(j / window), blocks counted from position 0; with
+    ``keep_first`` f > 0 the positions j < f stay visible whatever the window.
+    s = q.k * scale; with ``softcap`` c > 0, s <- c tanh(s / c);
+    score = s - r1[a] ln(1 + r2[a] (i - j)) + dist_bias[min(i - j, nd - 1), a]; weight =
+    softmax over the visible keys, or sigmoid(score + pb[a]) without normalisation.
+    ``sink`` (a score, softmax only): the softmax's denominator gains exp(sink), as if one
+    more key with that score and no value were always visible."""
     heads: int
     kv_heads: int
     dk: int
@@ -402,6 +486,9 @@ class WindowSpec:
     pb: Optional[torch.Tensor] = None     # fp32 [heads * maps] (sigmoid weights only)
     softcap: float = 0.0
     sink: Optional[float] = None
+    blocks: bool = False
+    keep_first: int = 0
+    dist_bias: Optional[torch.Tensor] = None   # fp32 [nd, heads * maps], :func:`distance_bias_table`
 
 
 def window_attention(q, k_cache, v_cache, seg: Segments, spec: WindowSpec, skip_from: int = 0,
@@ -416,26 +503,29 @@ def window_attention(q, k_cache, v_cache, seg: Segments, spec: WindowSpec, skip_
         native_mixers().window_attention(out, q, k_cache, v_cache, seg.start, seg.pos0, seg.kv_len,
                                          seg.block_tables, seg.num, seg.max_rows, sp.heads, sp.maps,
                                          sp.kv_heads, sp.dk, sp.dv, sp.window, sp.scale, sp.sigmoid,
-                                         sp.r1, sp.r2, sp.pb, skip_from, float(sp.softcap), sp.sink)
+                                         sp.r1, sp.r2, sp.pb, skip_from, float(sp.softcap), sp.sink,
+                                         bool(sp.blocks), int(sp.keep_first), sp.dist_bias)
         return out
     r = ref.window_attention(q, k_cache, v_cache, seg, sp.heads, sp.maps, sp.kv_heads, sp.dk, sp.dv,
-                             sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, sp.softcap, sp.sink)
+                             sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, sp.softcap, sp.sink,
+                             sp.blocks, sp.keep_first, sp.dist_bias)
     if out is not None:
         out.copy_(r)
         return out
     return r
 
 
-def band_weights(s, first_pos: int, key0: int, spec: WindowSpec, rep_rows: int):
+def band_weights(s, first_pos: int, key0: int, spec: WindowSpec, rep_rows: int, ext: int = 0):
     """Raw dot products fp32 [kv_heads*maps, rep*rows, keys] (the query heads that share
     a key head stacked along the rows, ``rep_rows`` = rows of one of them) -> attention
-    weights fp32, in place: row r of a head is position first_pos + r, column c is
-    position key0 + c."""
+    weights fp32, in place: row r of a head is position first_pos + r; the first ``ext``
+    columns are the positions 0 .. ext-1 (kept first tokens in front of the band), column
+    c >= ext is position key0 + c - ext."""
     sp = spec
     if s.is_cuda:
         native_mixers().band_weights(s, rep_rows, first_pos, key0, sp.heads, sp.maps, sp.kv_heads,
                                      sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, float(sp.softcap),
-                                     sp.sink)
+                                     sp.sink, bool(sp.blocks), int(sp.keep_first), int(ext), sp.dist_bias)
         return s
     g, rr, keys = s.shape
     rep = sp.heads // sp.kv_heads
@@ -443,14 +533,15 @@ def band_weights(s, first_pos: int, key0: int, spec: WindowSpec, rep_rows: int):
     v = s.view(sp.kv_heads, sp.maps, rep, rep_rows, keys).permute(0, 2, 1, 3, 4) \
         .reshape(sp.heads * sp.maps, rep_rows, keys)
     w = ref.band_weights(v, first_pos, key0, sp.window, sp.scale, sp.sigmoid, sp.r1, sp.r2, sp.pb, sp.softcap,
-                         sp.sink)
+                         sp.sink, sp.blocks, sp.keep_first, ext, sp.dist_bias)
     s.copy_(w.view(sp.kv_heads, rep, sp.maps, rep_rows, keys).permute(0, 2, 1, 3, 4).reshape(g, rr, keys))
     return s
 
 
 def window_attention_products(out, q, k_cache, v_cache, seg: Segments, spec: WindowSpec, min_rows: int):
     """Segments of ``min_rows`` rows or more as banded matrix products: a chunk of rows
-    [c0, c1) only sees the keys c0 - window + 1 .. c1 - 1, so per chunk and key head the
+    [c0, c1) only sees the keys c0 - window + 1 .. c1 - 1 (or from the start of c0's block;
+    plus the kept first positions, gathered in front of the band), so per chunk and key head the
     scores are one product with M = (query heads of the group) x rows, the weights come
     from :func:`band_weights` (fp32) and the sums are a second product with the value
     head.  Operands are fp32 (cached rows are widened), so scores, weights and sums are
@@ -475,20 +566,26 @@ def window_attention_products(out, q, k_cache, v_cache, seg: Segments, spec: Win
             c1 = min(n, c0 + step)
             rows = c1 - c0
             i0 = pos0[s] + c0
-            lo = max(0, i0 - sp.window + 1) if sp.window > 0 else 0
+            lo = ref.mask_first_key(i0, sp.window, sp.blocks)
+            ext = min(sp.keep_first, lo) if sp.window > 0 else 0
             hi = min(kv_len[s], pos0[s] + c1)
             b0, b1 = lo // bs, (hi + bs - 1) // bs
             blocks = seg.block_tables[s, b0:b1].long()
             off = lo - b0 * bs
             k = k_cache.index_select(0, blocks).view((b1 - b0) * bs, gk, sp.dk)[off:off + hi - lo].float()
             v = v_cache.index_select(0, blocks).view((b1 - b0) * bs, sp.kv_heads, sp.dv)[off:off + hi - lo].float()
+            if ext:
+                # the kept first positions 0 .. ext-1 lie before the band: their rows go in front
+                eb = seg.block_tables[s, :(ext + bs - 1) // bs].long()
+                k = torch.cat([k_cache.index_select(0, eb).view(-1, gk, sp.dk)[:ext].float(), k], 0)
+                v = torch.cat([v_cache.index_select(0, eb).view(-1, sp.kv_heads, sp.dv)[:ext].float(), v], 0)
             # q rows [rows, (g, r, m), dk] -> [(g, m), (r, rows), dk]
             qc = q[a + c0:a + c1].view(rows, sp.kv_heads, rep, sp.maps, sp.dk).permute(1, 3, 2, 0, 4) \
                 .reshape(gk, rep * rows, sp.dk)
             sc = torch.bmm(qc, k.permute(1, 2, 0))                       # [gk, rep*rows, keys]
-            band_weights(sc, i0, lo, sp, rows)
+            band_weights(sc, i0, lo, sp, rows, ext)
             # both maps of a group read the same value head: [G, maps*rep*rows, keys] x [G, keys, dv]
-            o = torch.bmm(sc.view(sp.kv_heads, sp.maps * rep * rows, hi - lo), v.transpose(0, 1))
+            o = torch.bmm(sc.view(sp.kv_heads, sp.maps * rep * rows, ext + hi - lo), v.transpose(0, 1))
             out[a + c0:a + c1] = o.view(sp.kv_heads, sp.maps, rep, rows, sp.dv).permute(3, 0, 2, 1, 4) \
                 .reshape(rows, sp.heads * sp.maps, sp.dv)
     return out
@@ -579,9 +676,18 @@ def gelu_glu(gu):
     """[gate | up] rows -> gelu_tanh(gate) * up."""
     if gu.is_cuda:
         out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
-        native_mixers().gelu_glu(out, gu)
+        native_mixers().gelu_glu(out, gu, False)
         return out
     return ref.gelu_glu(gu)
+
+
+def relu_glu(gu):
+    """[gate | up] rows -> relu(gate) * up."""
+    if gu.is_cuda:
+        out = torch.empty(gu.shape[0], gu.shape[1] // 2, dtype=gu.dtype, device=gu.device)
+        native_mixers().gelu_glu(out, gu, True)
+        return out
+    return ref.relu_glu(gu)
 
 
 def relu_sq(x):

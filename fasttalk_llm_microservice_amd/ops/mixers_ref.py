@@ -78,6 +78,38 @@ def add_rms_norm_rows(residual, y, wb, eps, add_vec, next_w, out_dtype, want_cas
     return out, cast
 
 
+def add_scaled_rms_norm_rows(residual, y1, y2, mult, next_w, eps, out_dtype):
+    if y1 is not None:
+        y = y1.float() if y2 is None else y1.float() + y2.float()
+        residual.add_(y * mult)
+    return (_rms(residual, eps) * next_w.float()).to(out_dtype) if next_w is not None else None
+
+
+def dual_rms_mean(a, b, wa, wb, eps, scale):
+    return scale * (_rms(a.float(), eps) * wa.float() + _rms(b.float(), eps) * wb.float())
+
+
+def pair_embed_add(x, ids, table, mul_prev: int, mul_cur: int, buckets: int, seg, last_tok):
+    start = seg.start.tolist()
+    tab = table.float()
+    for s in range(seg.num):
+        a, b = start[s], start[s + 1]
+        slot = int(seg.slot[s])
+        if b == a or slot < 0:
+            continue
+        cur = ids[a:b].long()
+        first = torch.full((1,), -1, dtype=torch.long) if int(seg.pos0[s]) <= 0 else last_tok[slot].long().view(1)
+        prev = torch.cat([first.to(cur.device), cur[:-1]])
+        rows = torch.where(prev < 0, torch.full_like(cur, buckets), (prev * mul_prev + cur * mul_cur) % buckets)
+        x[a:b] += tab[rows]
+        last_tok[slot] = cur[-1].to(last_tok.dtype)
+    return x
+
+
+def sigmoid_gate(o, g, out_dtype):
+    return (o.float() * torch.sigmoid(g.float())).to(out_dtype)
+
+
 def scale_frequencies(f, factor: float, low: float, high: float, original: float):
     """Rotary frequencies stretched for long contexts.  With t_i = original * f_i / (2 pi)
     (how many turns pair i makes over ``original`` positions): f_i stays for t_i > high,
@@ -89,16 +121,59 @@ def scale_frequencies(f, factor: float, low: float, high: float, original: float
     return torch.where(wl < original / high, f, torch.where(wl > original / low, f / factor, mid))
 
 
-def rope_table(max_pos: int, dims: int, base: float, device=None, scaling=None):
+def ramp_frequencies(dims: int, base: float, factor: float, original: float, fast: float, slow: float):
+    """Rotary frequencies divided by ``factor`` along a linear ramp over the pair index,
+    and the factor that goes with them on cos and sin.  With
+    where(t) = dims ln(original / (2 pi t)) / (2 ln base) -- the (fractional) pair index
+    that makes t turns over ``original`` positions -- lo = max(floor(where(fast)), 0),
+    hi = min(ceil(where(slow)), dims - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1):
+    f_i' = r_i f_i / factor + (1 - r_i) f_i; cos and sin are multiplied by
+    0.1 ln(factor) + 1.  Evaluated in double precision on the host; returns (fp32 [dims/2],
+    float)."""
+    where = lambda t: dims * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(base))   # noqa: E731
+    lo = max(math.floor(where(fast)), 0)
+    hi = min(math.ceil(where(slow)), dims - 1)
+    f = []
+    for i in range(dims // 2):
+        fi = float(base) ** (-2.0 * i / dims)
+        r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        f.append(fi / factor * r + fi * (1.0 - r))
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
+def rope_table(max_pos: int, dims: int, base: float, device=None, scaling=None, ramp=None):
     """fp32 [max_pos, dims] = [cos | sin]; frequencies, angles and their cos / sin are
     all evaluated in fp32 (angle = float(p) * f_i, f_i = base^(-2i/dims));
-    ``scaling``: (factor, low, high, original) for :func:`scale_frequencies`."""
+    ``scaling``: (factor, low, high, original) for :func:`scale_frequencies`; ``ramp``:
+    (factor, original, fast, slow) for :func:`ramp_frequencies`, whose factor on cos and
+    sin is folded into the table."""
     i = torch.arange(dims // 2, dtype=torch.float32)
     f = torch.tensor(float(base), dtype=torch.float32) ** (-2.0 * i / dims)
+    mult = 1.0
     if scaling is not None:
         f = scale_frequencies(f, *[float(v) for v in scaling])
+    if ramp is not None:
+        f, mult = ramp_frequencies(dims, float(base), *[float(v) for v in ramp])
     a = torch.arange(max_pos, dtype=torch.float32)[:, None] * f[None]
-    return torch.cat([a.cos(), a.sin()], -1).to(device)
+    t = torch.cat([a.cos(), a.sin()], -1)
+    if mult != 1.0:
+        t = t * torch.tensor(mult, dtype=torch.float32)
+    return t.to(device)
+
+
+def distance_bias_table(rel, reach: int):
+    """fp32 [reach + 1, heads]: row n is the row of ``rel`` [B, heads] that distance n falls
+    into -- n itself below B // 2, then logarithmic steps up to ``reach``:
+    min(B - 1, B//2 + floor(ln(n / (B//2)) / ln(reach / (B//2)) (B - B//2))).  Every distance
+    of ``reach`` or more falls into the last row, so a kernel clamps the distance to
+    ``reach`` and reads this table.  The steps are evaluated in double precision."""
+    B = rel.shape[0]
+    half = B // 2
+    if reach <= half or half < 1:
+        raise ValueError("the distance bias needs 1 <= rows // 2 < reach")
+    idx = [n if n < half else min(B - 1, half + math.floor(math.log(n / half) / math.log(reach / half) * (B - half)))
+           for n in range(reach + 1)]
+    return rel.float()[torch.tensor(idx, dtype=torch.long, device=rel.device)].contiguous()
 
 
 def _rope(x, cs, dims):
@@ -163,10 +238,33 @@ def gated_delta_rule(qkv, a, b, a_log, dt_bias, state, seg, heads, kv_heads, dk,
     return o.view(t, heads * dv)
 
 
-def head_rms_gate(o, w, gate_pre, eps, heads, dv, out_dtype):
+def gated_linear_attention(qkv, a, a_bias, tau, state, seg, heads, dk, dv):
+    t = qkv.shape[0]
+    n = heads * dk
+    q = qkv[:, :n].float().view(t, heads, dk) * torch.tensor(float(dk), dtype=torch.float32) ** -0.5
+    k = qkv[:, n:2 * n].float().view(t, heads, dk)
+    v = qkv[:, 2 * n:2 * n + heads * dv].float().view(t, heads, dv)
+    g = torch.exp(F.logsigmoid(a.float() + a_bias.float()) / float(tau)).view(t, heads, dk)
+    o = torch.zeros(t, heads, dv, dtype=torch.float32, device=qkv.device)
+    start = seg.start.tolist()
+    for s in range(seg.num):
+        slot = int(seg.slot[s])
+        if slot < 0:
+            continue
+        S = state[slot] if int(seg.pos0[s]) > 0 else torch.zeros_like(state[slot])
+        for r in range(start[s], start[s + 1]):
+            S = g[r][:, :, None] * S + k[r][:, :, None] * v[r][:, None, :]
+            o[r] = torch.einsum("hkv,hk->hv", S, q[r])
+        if start[s + 1] > start[s]:
+            state[slot] = S
+    return o.view(t, heads * dv)
+
+
+def head_rms_gate(o, w, gate_pre, eps, heads, dv, out_dtype, silu=False):
     t = o.shape[0]
     x = o.view(t, heads, dv)
-    y = _rms(x, eps) * w.float() * torch.sigmoid(gate_pre.float().view(t, heads, dv))
+    g = gate_pre.float().reshape(t, heads, dv)
+    y = _rms(x, eps) * w.float() * (g * torch.sigmoid(g) if silu else torch.sigmoid(g))
     return y.view(t, heads * dv).to(out_dtype)
 
 
@@ -314,6 +412,8 @@ def attn_prep(qkv, nq, nk, q_norm_w, k_norm_w, eps, table, rot_dims, head_dim, p
         cs = table[positions[:t].long()]
         q = _rope(q.reshape(t, -1, head_dim).transpose(0, 1), cs, rot_dims).transpose(0, 1).reshape(t, nq)
         k = _rope(k.reshape(t, -1, head_dim).transpose(0, 1), cs, rot_dims).transpose(0, 1).reshape(t, nk)
+    if k_cache is None:
+        return q.contiguous()
     slots = slot_mapping[:t].long()
     keep = slots >= 0
     if keep.any():
@@ -353,21 +453,39 @@ def conv_attn_prep(qkv, nq, nk, conv_w, conv_state, seg, q_norm_w, k_norm_w, eps
     return q.contiguous()
 
 
-def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb, softcap=0.0, sink=None):
+def mask_first_key(i: int, window: int, blocks: bool) -> int:
+    """The first position that position i sees through its window (or its block)."""
+    if window <= 0:
+        return 0
+    return (i // window) * window if blocks else max(0, i - window + 1)
+
+
+def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb, softcap=0.0, sink=None,
+                 blocks=False, keep_first=0, ext=0, dist_bias=None):
     """s fp32 [heads, rows, keys] raw dot products -> attention weights: row r is position
-    first_pos + r, column c is position key0 + c, visible iff 0 <= i - j (< window)."""
+    i = first_pos + r; the first ``ext`` columns are positions 0 .. ext-1 and column
+    c >= ext is position j = key0 + c - ext.  Visible iff j <= i and (i - j < window, or
+    with ``blocks`` floor(i / window) = floor(j / window), or j < keep_first); window 0:
+    every earlier key.  ``dist_bias`` fp32 [nd, heads] adds dist_bias[min(i - j, nd - 1), h]."""
     heads, rows, keys = s.shape
-    dist = (first_pos + torch.arange(rows, device=s.device))[:, None] - \
-        (key0 + torch.arange(keys, device=s.device))[None, :]
+    col = torch.arange(keys, device=s.device)
+    jpos = torch.where(col < ext, col, key0 + col - ext)
+    ipos = first_pos + torch.arange(rows, device=s.device)
+    dist = ipos[:, None] - jpos[None, :]
     vis = dist >= 0
     if window > 0:
-        vis &= dist < window
+        inside = (ipos[:, None] // window == jpos[None, :] // window) if blocks else dist < window
+        if keep_first > 0:
+            inside = inside | (jpos[None, :] < keep_first)
+        vis = vis & inside
     z = s * scale
     if softcap:
         z = softcap * torch.tanh(z / softcap)
     if r1 is not None:
         z = z - r1.float()[:, None, None] * torch.log(1.0 + r2.float()[:, None, None]
                                                       * dist.clamp_min(0).float()[None])
+    if dist_bias is not None:
+        z = z + dist_bias.float()[dist.clamp(0, dist_bias.shape[0] - 1)].permute(2, 0, 1)
     if sigmoid:
         if pb is not None:
             z = z + pb.float()[:, None, None]
@@ -381,7 +499,7 @@ def band_weights(s, first_pos, key0, window, scale, sigmoid, r1, r2, pb, softcap
 
 
 def window_attention(q, k_cache, v_cache, seg, heads, maps, kv_heads, dk, dv, window, scale, sigmoid,
-                     r1, r2, pb, softcap=0.0, sink=None):
+                     r1, r2, pb, softcap=0.0, sink=None, blocks=False, keep_first=0, dist_bias=None):
     """q fp32 [T, heads*maps*dk]; caches [blocks, bs, kv_heads*maps*dk] / [blocks, bs,
     kv_heads*dv]; returns fp32 [T, heads*maps, dv]."""
     t = q.shape[0]
@@ -399,14 +517,17 @@ def window_attention(q, k_cache, v_cache, seg, heads, maps, kv_heads, dk, dv, wi
         if b == a or n == 0:
             continue
         p0 = int(seg.pos0[s])
-        lo = max(0, p0 - window + 1) if window > 0 else 0
+        lo = mask_first_key(p0, window, blocks)
+        ext = min(keep_first, lo) if window > 0 else 0
         nblk = (n + bs - 1) // bs
-        blocks = seg.block_tables[s, :nblk].long()
-        k = k_cache[blocks].reshape(nblk * bs, -1)[lo:n].float().view(n - lo, kv_heads * maps, dk)
-        v = v_cache[blocks].reshape(nblk * bs, -1)[lo:n].float().view(n - lo, kv_heads, dv)
+        pages = seg.block_tables[s, :nblk].long()
+        keys = torch.cat([torch.arange(ext), torch.arange(lo, n)]).to(k_cache.device)
+        k = k_cache[pages].reshape(nblk * bs, -1)[keys].float().view(keys.numel(), kv_heads * maps, dk)
+        v = v_cache[pages].reshape(nblk * bs, -1)[keys].float().view(keys.numel(), kv_heads, dv)
         qs = q[a:b].view(b - a, hq, dk)
         sc = torch.einsum("thd,jhd->htj", qs, k[:, khead])
-        w = band_weights(sc, p0, lo, window, scale, sigmoid, r1, r2, pb, softcap, sink)
+        w = band_weights(sc, p0, lo, window, scale, sigmoid, r1, r2, pb, softcap, sink, blocks, keep_first, ext,
+                         dist_bias)
         out[a:b] = torch.einsum("htj,jhd->thd", w, v[:, vhead])
     return out
 
@@ -449,6 +570,11 @@ def gate_group_norm(y, z, w, eps, groups, out_dtype):
     v = y * (zf * torch.sigmoid(zf))
     v = _rms(v.view(t, groups, inner // groups), eps).view(t, inner) * w.float()
     return v.to(out_dtype)
+
+
+def relu_glu(gu):
+    ff = gu.shape[1] // 2
+    return (torch.relu(gu[:, :ff].float()) * gu[:, ff:].float()).to(gu.dtype)
 
 
 def gelu_glu(gu):
