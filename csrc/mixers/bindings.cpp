@@ -28,7 +28,21 @@ int mx_conv_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int 
 int mx_moe_top_logits(int* idx, float* wts, const float* z, long rows, int experts, int top, hipStream_t s);
 int mx_moe_route_top_logits(int* idx, float* wts, const void* h, int bf16, long h_stride, const float* router,
                             const float* bias, long rows, int experts, int width, int top, hipStream_t s);
-int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, hipStream_t s);
+int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, int relu, hipStream_t s);
+int mx_gla_max_dk();
+int mx_gla_scan(float* o, const void* qkv, int bf16, long qkv_stride, const void* a, long a_stride,
+                const float* a_bias, float tau, float* state, const int* start, const int* pos0, const int* slot,
+                int num_segs, int max_rows, int heads, int dk, int dv, int num_slots, hipStream_t s);
+int mx_pair_embed_add(float* x, const int* ids, const void* table, int bf16, int rows, int width, long mul_prev,
+                      long mul_cur, int buckets, const int* start, const int* pos0, const int* slot, int num_segs,
+                      int* last_tok, int num_slots, const void* embed, int vocab, float scale, hipStream_t s);
+int mx_add_scaled_rms_norm(float* x, const void* y1, int y1_bf16, long y1_stride, const void* y2, int y2_bf16,
+                           long y2_stride, float mult, const float* next_w, void* out, int out_bf16, int rows,
+                           int width, float eps, hipStream_t s);
+int mx_dual_rms_mean(float* out, const void* a, long a_stride, const void* b, long b_stride, int bf16,
+                     const float* wa, const float* wb, int rows, int width, float eps, float scale, hipStream_t s);
+int mx_sigmoid_gate(void* out, int out_bf16, const float* o, const void* g, int g_bf16, long g_stride, long rows,
+                    int n, hipStream_t s);
 int mx_attn_prep(float* q_out, const void* qkv, int bf16, long stride, int nq, int nk, int nv, const float* wq,
                  const float* wk, float eps, const float* table, int table_rows, int rot_dims, int head_dim,
                  const int* positions, const int* slots, void* k_cache, void* v_cache, int cache_bf16,
@@ -38,10 +52,12 @@ int mx_window_attention(float* out, const float* q, const void* k_cache, const v
                         const int* start, const int* pos0, const int* kv_len, const int* bt, int bt_stride,
                         int num_segs, long total_rows, int heads, int maps, int kv_heads, int dk, int dv, int window,
                         float scale, int sigmoid, const float* r1, const float* r2, const float* pb, int block_size,
-                        int num_blocks, int skip_from, float softcap, int has_sink, float sink, hipStream_t s);
+                        int num_blocks, int skip_from, float softcap, int has_sink, float sink, int blocks,
+                        int keep_first, const float* dist_bias, int nd, hipStream_t s);
 int mx_band_weights(float* S, int gk, int rep_rows_total, int rows, int keys, int first_pos, int key0, int heads,
                     int maps, int kv_heads, int window, float scale, int sigmoid, const float* r1, const float* r2,
-                    const float* pb, float softcap, int has_sink, float sink, hipStream_t s);
+                    const float* pb, float softcap, int has_sink, float sink, int blocks, int keep_first, int ext,
+                    const float* dist_bias, int nd, hipStream_t s);
 int mx_diff_combine(void* out, int out_bf16, const float* a, const void* gate, int gate_bf16, long gate_stride,
                     long rows, int heads, int dv, float lam, float post, float eps, hipStream_t s);
 int mx_ssd_max_state();
@@ -55,7 +71,7 @@ int mx_add_rms_norm(float* x, const void* y, int y_bf16, long y_stride, const fl
                     const float* next_w, void* out, void* cast, int out_bf16, int rows, int width, float eps,
                     hipStream_t s);
 int mx_head_rms_gate(void* out, int out_bf16, const float* o, const float* w, const void* gate, int gate_bf16,
-                     long gate_stride, long rows, int heads, int dv, float eps, hipStream_t s);
+                     long gate_stride, long rows, int heads, int dv, float eps, int silu, hipStream_t s);
 int mx_relu_sq(void* x, int bf16, long n, hipStream_t s);
 int mx_clamp_swiglu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, float limit,
                     hipStream_t s);
@@ -111,6 +127,8 @@ bool is_act(const Tensor& t) { return t.scalar_type() == at::kFloat || t.scalar_
 int bf(const Tensor& t) { return t.scalar_type() == at::kBFloat16 ? 1 : 0; }
 
 void chk(int rc, const char* what) { TORCH_CHECK(rc == 0, what, " failed (", rc, ")"); }
+
+const float* opt_f32(const c10::optional<at::Tensor>& t, int64_t n, const char* what);
 
 void check_f32(const Tensor& t, const char* n) {
   TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), n, ": fp32 contiguous GPU tensor");
@@ -225,7 +243,7 @@ void add_rms_norm(Tensor x, OptT y, OptT wb, OptT add_vec, OptT next_w, OptT out
                       (int)width, (float)eps, stream()), "add_rms_norm");
 }
 
-void head_rms_gate(Tensor out, Tensor o, Tensor w, Tensor gate, double eps, int64_t heads, int64_t dv) {
+void head_rms_gate(Tensor out, Tensor o, Tensor w, Tensor gate, double eps, int64_t heads, int64_t dv, bool silu) {
   check_f32(o, "o");
   check_f32(w, "w");
   check_rows(gate, "gate");
@@ -234,7 +252,8 @@ void head_rms_gate(Tensor out, Tensor o, Tensor w, Tensor gate, double eps, int6
   TORCH_CHECK(out.is_cuda() && is_act(out) && out.is_contiguous() && out.sizes() == o.sizes() &&
               bf(out) == bf(gate), "out");
   chk(mx_head_rms_gate(out.data_ptr(), bf(out), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(),
-                       bf(gate), gate.stride(0), o.size(0), (int)heads, (int)dv, (float)eps, stream()),
+                       bf(gate), gate.stride(0), o.size(0), (int)heads, (int)dv, (float)eps, silu ? 1 : 0,
+                       stream()),
       "head_rms_gate");
 }
 
@@ -359,6 +378,102 @@ void gated_delta_rule(Tensor o, Tensor qkv, Tensor a, Tensor b, Tensor a_log, Te
                     beta.data_ptr<float>(), qkv.data_ptr(), bf(qkv), qkv.stride(0), state.data_ptr<float>(),
                     start.data_ptr<int>(), pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs, (int)heads,
                     (int)kv_heads, (int)dk, (int)dv, (int)state.size(0), stream()), "delta_rule");
+}
+
+void gated_linear_attention(Tensor o, Tensor qkv, Tensor a, Tensor a_bias, double tau, Tensor state, Tensor start,
+                            Tensor pos0, Tensor slot, int64_t num_segs, int64_t max_rows, int64_t heads, int64_t dk,
+                            int64_t dv) {
+  check_f32(o, "o");
+  check_rows(qkv, "qkv");
+  check_rows(a, "a");
+  check_f32(a_bias, "a_bias");
+  check_f32(state, "state");
+  const int64_t t = qkv.size(0);
+  TORCH_CHECK(heads >= 1 && dk >= 1 && dk <= mx_gla_max_dk() && dv >= 1 && tau > 0, "linear attention sizes");
+  TORCH_CHECK(qkv.size(1) >= heads * (2 * dk + dv) && a.size(0) == t && a.size(1) == heads * dk &&
+              a_bias.numel() == heads * dk && o.numel() == t * heads * dv && a.scalar_type() == qkv.scalar_type(),
+              "linear attention shapes");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == heads && state.size(2) == dk && state.size(3) == dv, "state");
+  check_segs(start, pos0, slot, num_segs);
+  TORCH_CHECK(start.numel() >= num_segs + 1, "segments");
+  chk(mx_gla_scan(o.data_ptr<float>(), qkv.data_ptr(), bf(qkv), qkv.stride(0), a.data_ptr(), a.stride(0),
+                  a_bias.data_ptr<float>(), (float)tau, state.data_ptr<float>(), start.data_ptr<int>(),
+                  pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs, (int)std::max<int64_t>(max_rows, 0),
+                  (int)heads, (int)dk, (int)dv, (int)state.size(0), stream()), "linear attention");
+}
+
+void pair_embed_add(Tensor x, Tensor ids, Tensor table, int64_t mul_prev, int64_t mul_cur, int64_t buckets,
+                    Tensor start, Tensor pos0, Tensor slot, int64_t num_segs, Tensor last_tok, OptT embed,
+                    double scale) {
+  check_f32(x, "residual");
+  if (embed)
+    TORCH_CHECK(embed->is_cuda() && embed->is_contiguous() && embed->dim() == 2 && embed->size(1) == x.size(1) &&
+                embed->scalar_type() == table.scalar_type(), "embedding table");
+  check_i32(ids, "ids");
+  check_i32(last_tok, "last tokens");
+  TORCH_CHECK(table.is_cuda() && is_act(table) && table.is_contiguous() && table.dim() == 2, "table");
+  TORCH_CHECK(x.dim() == 2 && x.size(0) == ids.numel() && x.size(1) == table.size(1) && buckets >= 1 &&
+              table.size(0) == buckets + 1 && mul_prev >= 0 && mul_cur >= 0, "pair_embed_add shapes");
+  check_segs(start, pos0, slot, num_segs);
+  chk(mx_pair_embed_add(x.data_ptr<float>(), ids.data_ptr<int>(), table.data_ptr(), bf(table), (int)ids.numel(),
+                        (int)table.size(1), (long)mul_prev, (long)mul_cur, (int)buckets, start.data_ptr<int>(),
+                        pos0.data_ptr<int>(), slot.data_ptr<int>(), (int)num_segs, last_tok.data_ptr<int>(),
+                        (int)last_tok.numel(), embed ? embed->data_ptr() : nullptr, embed ? (int)embed->size(0) : 0,
+                        (float)scale, stream()), "pair_embed_add");
+}
+
+void add_scaled_rms_norm(Tensor x, OptT y1, OptT y2, double mult, OptT next_w, OptT out, double eps) {
+  check_f32(x, "residual");
+  TORCH_CHECK(x.dim() == 2, "residual 2-D");
+  const int64_t rows = x.size(0), width = x.size(1);
+  TORCH_CHECK((bool)next_w == (bool)out && (y1 || (!y2 && out)), "add_scaled_rms_norm arguments");
+  const void *p1 = nullptr, *p2 = nullptr;
+  int b1 = 0, b2 = 0;
+  long s1 = 0, s2 = 0;
+  if (y1) {
+    check_rows(*y1, "y1");
+    TORCH_CHECK(y1->size(0) == rows && y1->size(1) == width, "y1 shape");
+    p1 = y1->data_ptr(); b1 = bf(*y1); s1 = y1->stride(0);
+  }
+  if (y2) {
+    check_rows(*y2, "y2");
+    TORCH_CHECK(y2->size(0) == rows && y2->size(1) == width, "y2 shape");
+    p2 = y2->data_ptr(); b2 = bf(*y2); s2 = y2->stride(0);
+  }
+  void* op = nullptr;
+  int obf = 0;
+  if (out) {
+    TORCH_CHECK(out->is_cuda() && out->is_contiguous() && is_act(*out) && out->sizes() == x.sizes(), "out");
+    op = out->data_ptr();
+    obf = bf(*out);
+  }
+  chk(mx_add_scaled_rms_norm(x.data_ptr<float>(), p1, b1, s1, p2, b2, s2, (float)mult,
+                             opt_f32(next_w, width, "next norm weight"), op, obf, (int)rows, (int)width, (float)eps,
+                             stream()), "add_scaled_rms_norm");
+}
+
+void dual_rms_mean(Tensor out, Tensor a, Tensor b, Tensor wa, Tensor wb, double eps, double scale) {
+  check_f32(out, "out");
+  check_rows(a, "a");
+  check_rows(b, "b");
+  check_f32(wa, "wa");
+  check_f32(wb, "wb");
+  const int64_t rows = a.size(0), width = a.size(1);
+  TORCH_CHECK(b.sizes() == a.sizes() && b.scalar_type() == a.scalar_type() && out.dim() == 2 && out.size(0) == rows &&
+              out.size(1) == width && wa.numel() == width && wb.numel() == width, "dual_rms_mean shapes");
+  chk(mx_dual_rms_mean(out.data_ptr<float>(), a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bf(a),
+                       wa.data_ptr<float>(), wb.data_ptr<float>(), (int)rows, (int)width, (float)eps, (float)scale,
+                       stream()), "dual_rms_mean");
+}
+
+void sigmoid_gate(Tensor out, Tensor o, Tensor g) {
+  check_f32(o, "o");
+  check_rows(g, "g");
+  TORCH_CHECK(o.dim() == 2 && g.size(0) == o.size(0) && g.size(1) == o.size(1), "sigmoid_gate shapes");
+  TORCH_CHECK(out.is_cuda() && is_act(out) && out.is_contiguous() && out.sizes() == o.sizes() && bf(out) == bf(g),
+              "out");
+  chk(mx_sigmoid_gate(out.data_ptr(), bf(out), o.data_ptr<float>(), g.data_ptr(), bf(g), g.stride(0), o.size(0),
+                      (int)o.size(1), stream()), "sigmoid_gate");
 }
 
 void latent_kv_write(Tensor dkv, Tensor w, double eps, Tensor table, int64_t dims, Tensor positions,
@@ -502,12 +617,13 @@ void moe_pairs(Tensor out, Tensor h, Tensor idx, Tensor wts, Tensor wgu, Tensor 
                    (int)width, (float)limit, relu_sq ? 1 : 0, stream()), "moe_pairs");
 }
 
-void gelu_glu(Tensor out, Tensor gu) {
+void gelu_glu(Tensor out, Tensor gu, bool relu) {
   check_rows(gu, "gu");
   const int64_t ff = gu.size(1) / 2;
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.scalar_type() == gu.scalar_type() && out.dim() == 2 &&
               out.size(0) == gu.size(0) && out.size(1) == ff && ff >= 1 && gu.size(1) == 2 * ff, "out");
-  chk(mx_gelu_glu(out.data_ptr(), gu.data_ptr(), bf(gu), gu.stride(0), gu.size(0), (int)ff, stream()), "gelu_glu");
+  chk(mx_gelu_glu(out.data_ptr(), gu.data_ptr(), bf(gu), gu.stride(0), gu.size(0), (int)ff, relu ? 1 : 0, stream()),
+      "gelu_glu");
 }
 
 const float* opt_f32(const OptT& t, int64_t n, const char* what) {
@@ -524,15 +640,35 @@ void check_cache(const Tensor& c, int64_t row, const char* n) {
 }
 
 void attn_prep(Tensor q, Tensor qkv, int64_t nq, int64_t nk, OptT wq, OptT wk, double eps, OptT table,
-               int64_t rot_dims, int64_t head_dim, Tensor positions, Tensor slots, Tensor k_cache, Tensor v_cache) {
+               int64_t rot_dims, int64_t head_dim, Tensor positions, Tensor slots, OptT k_cache_, OptT v_cache_) {
   check_f32(q, "q");
   check_rows(qkv, "qkv");
   check_i32(positions, "positions");
   check_i32(slots, "slot_mapping");
   const int64_t t = qkv.size(0), nv = qkv.size(1) - nq - nk;
-  TORCH_CHECK(nq >= 1 && nk >= 1 && nv >= 1 && head_dim >= 1 && nq % head_dim == 0 && nk % head_dim == 0 &&
+  TORCH_CHECK(nq >= 1 && head_dim >= 1 && nq % head_dim == 0 && nk % head_dim == 0 &&
               rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= head_dim && q.numel() == t * nq &&
               positions.numel() >= t && slots.numel() >= t, "attn_prep shapes");
+  if (!k_cache_ || !v_cache_) {
+    // queries alone (a layer that attends to another layer's keys and values)
+    TORCH_CHECK(!k_cache_ && !v_cache_ && nk == 0 && nv == 0 && !wk, "attn_prep: no caches goes with rows of q alone");
+    const float* tq = nullptr;
+    int64_t tr = 0;
+    if (table && rot_dims > 0) {
+      check_f32(*table, "rope table");
+      TORCH_CHECK(table->dim() == 2 && table->size(1) == rot_dims, "rope table shape");
+      tq = table->data_ptr<float>();
+      tr = table->size(0);
+    }
+    chk(mx_attn_prep(q.data_ptr<float>(), qkv.data_ptr(), bf(qkv), qkv.stride(0), (int)nq, 0, 0,
+                     opt_f32(wq, nq, "q norm"), nullptr, (float)eps, tq, (int)tr, (int)rot_dims, (int)head_dim,
+                     positions.data_ptr<int>(), slots.data_ptr<int>(), nullptr, nullptr, bf(qkv), 0, t, stream()),
+        "attn_prep");
+    return;
+  }
+  const Tensor& k_cache = *k_cache_;
+  const Tensor& v_cache = *v_cache_;
+  TORCH_CHECK(nk >= 1 && nv >= 1, "attn_prep shapes");
   check_cache(k_cache, nk, "k_cache");
   check_cache(v_cache, nv, "v_cache");
   TORCH_CHECK(k_cache.scalar_type() == v_cache.scalar_type() && k_cache.size(0) == v_cache.size(0) &&
@@ -581,9 +717,16 @@ void conv_attn_prep(Tensor q, Tensor qkv, int64_t nq, int64_t nk, Tensor conv_w,
 void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor start, Tensor pos0, Tensor kv_len,
                       Tensor bt, int64_t num_segs, int64_t max_rows, int64_t heads, int64_t maps, int64_t kv_heads,
                       int64_t dk, int64_t dv, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb,
-                      int64_t skip_from, double softcap, c10::optional<double> sink) {
+                      int64_t skip_from, double softcap, c10::optional<double> sink, bool blocks,
+                      int64_t keep_first, OptT dist_bias) {
   check_f32(out, "out");
   check_f32(q, "q");
+  TORCH_CHECK(keep_first >= 0 && (!blocks || window >= 1), "window attention mask");
+  if (dist_bias) {
+    check_f32(*dist_bias, "distance bias");
+    TORCH_CHECK(dist_bias->dim() == 2 && dist_bias->size(0) >= 1 && dist_bias->size(1) == heads * maps,
+                "distance bias [distances, heads]");
+  }
   TORCH_CHECK(heads >= 1 && maps >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && dk >= 1 && dv >= 1 &&
               dv <= mx_window_max_dv(), "window attention sizes");
   const int64_t hq = heads * maps, t = q.size(0);
@@ -601,14 +744,24 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache, Tens
                           bt.data_ptr<int>(), (int)bt.size(1), (int)num_segs, t, (int)heads, (int)maps, (int)kv_heads,
                           (int)dk, (int)dv, (int)window, (float)scale, sigmoid ? 1 : 0, opt_f32(r1, hq, "r1"),
                           opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), (int)k_cache.size(1), (int)k_cache.size(0),
-                          (int)skip_from, (float)softcap, sink ? 1 : 0, sink ? (float)*sink : 0.f, stream()),
+                          (int)skip_from, (float)softcap, sink ? 1 : 0, sink ? (float)*sink : 0.f, blocks ? 1 : 0,
+                          (int)keep_first, dist_bias ? dist_bias->data_ptr<float>() : nullptr,
+                          dist_bias ? (int)dist_bias->size(0) : 0, stream()),
       "window_attention");
 }
 
 void band_weights(Tensor S, int64_t rows, int64_t first_pos, int64_t key0, int64_t heads, int64_t maps,
                   int64_t kv_heads, int64_t window, double scale, bool sigmoid, OptT r1, OptT r2, OptT pb,
-                  double softcap, c10::optional<double> sink) {
+                  double softcap, c10::optional<double> sink, bool blocks, int64_t keep_first, int64_t ext,
+                  OptT dist_bias) {
   check_f32(S, "S");
+  TORCH_CHECK(keep_first >= 0 && ext >= 0 && ext <= key0 && ext <= S.size(2) && (!blocks || window >= 1),
+              "band_weights mask");
+  if (dist_bias) {
+    check_f32(*dist_bias, "distance bias");
+    TORCH_CHECK(dist_bias->dim() == 2 && dist_bias->size(0) >= 1 && dist_bias->size(1) == heads * maps,
+                "distance bias [distances, heads]");
+  }
   TORCH_CHECK(S.dim() == 3 && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && maps >= 1 &&
               S.size(0) == kv_heads * maps && rows >= 1 && S.size(1) == heads / kv_heads * rows && first_pos >= 0 &&
               key0 >= 0, "band_weights shapes");
@@ -617,7 +770,9 @@ void band_weights(Tensor S, int64_t rows, int64_t first_pos, int64_t key0, int64
   chk(mx_band_weights(S.data_ptr<float>(), (int)S.size(0), (int)S.size(1), (int)rows, (int)S.size(2), (int)first_pos,
                       (int)key0, (int)heads, (int)maps, (int)kv_heads, (int)window, (float)scale, sigmoid ? 1 : 0,
                       opt_f32(r1, hq, "r1"), opt_f32(r2, hq, "r2"), opt_f32(pb, hq, "pb"), (float)softcap, sink ? 1 : 0,
-                      sink ? (float)*sink : 0.f, stream()), "band_weights");
+                      sink ? (float)*sink : 0.f, blocks ? 1 : 0, (int)keep_first, (int)ext,
+                      dist_bias ? dist_bias->data_ptr<float>() : nullptr, dist_bias ? (int)dist_bias->size(0) : 0,
+                      stream()), "band_weights");
 }
 
 void diff_combine(Tensor out, Tensor a, Tensor gate, double lam, double post, double eps, int64_t heads, int64_t dv) {
@@ -688,6 +843,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("scale_add_rows", &scale_add_rows);
   m.def("short_conv_silu", &short_conv_silu);
   m.def("gated_delta_rule", &gated_delta_rule);
+  m.def("gated_linear_attention", &gated_linear_attention);
+  m.def("pair_embed_add", &pair_embed_add);
+  m.def("add_scaled_rms_norm", &add_scaled_rms_norm);
+  m.def("dual_rms_mean", &dual_rms_mean);
+  m.def("sigmoid_gate", &sigmoid_gate);
   m.def("latent_kv_write", &latent_kv_write);
   m.def("latent_q_rope", &latent_q_rope);
   m.def("latent_attention", &latent_attention);

@@ -28,6 +28,124 @@ __global__ void embed_rows_kernel(float* __restrict__ out, const int* __restrict
   }
 }
 
+// a value of a row that is fp32 or bf16, decided at run time (uniform over the launch)
+__device__ __forceinline__ float ldx(const void* p, int bf16, long i) {
+  return bf16 ? ft::bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+}
+
+// x (fp32 residual) = embed[cur] * scale + table[hash] per row (without `embed`: x +=
+// table[hash]), hash = (prev * mul_prev + cur * mul_cur) mod
+// buckets with prev the token before the row's own in its sequence: the row above within a
+// segment, last_tok[slot] for a segment's first row (pos0 > 0), and for a sequence's first
+// token row `buckets` instead.  One workgroup per row; pair_last_kernel stores each
+// segment's last token afterwards (a second launch: another row of the segment may still
+// be reading the old one).
+template <typename T>
+__global__ void pair_embed_add_kernel(float* __restrict__ x, const int* __restrict__ ids,
+                                      const T* __restrict__ table, int width, long mul_prev, long mul_cur,
+                                      int buckets, const int* __restrict__ start, const int* __restrict__ pos0,
+                                      const int* __restrict__ slot, int num_segs, const int* __restrict__ last_tok,
+                                      int num_slots, const T* __restrict__ embed, int vocab, float scale) {
+  const int row = blockIdx.x;
+  if (embed != nullptr) {                 // every row gets its embedding row, padding rows too
+    int id = ids[row];
+    if (id < 0 || id >= vocab) id = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+      x[(long)row * width + i] = ld(embed, (long)id * width + i) * scale;
+  }
+  if (row >= start[num_segs]) return;
+  int lo_s = 0, hi_s = num_segs;
+  while (hi_s - lo_s > 1) {
+    const int mid = (lo_s + hi_s) >> 1;
+    if (start[mid] <= row) lo_s = mid; else hi_s = mid;
+  }
+  const int sg = lo_s;
+  const int sl = slot[sg];
+  if (sl < 0 || sl >= num_slots) return;
+  long prev;
+  if (row > start[sg]) prev = ids[row - 1];
+  else prev = pos0[sg] > 0 ? last_tok[sl] : -1;
+  long idx = buckets;
+  if (prev >= 0) {
+    idx = (prev * mul_prev + (long)ids[row] * mul_cur) % buckets;
+    if (idx < 0) idx += buckets;
+  }
+  for (int i = threadIdx.x; i < width; i += blockDim.x) x[(long)row * width + i] += ld(table, idx * width + i);
+}
+
+__global__ void pair_last_kernel(const int* __restrict__ ids, const int* __restrict__ start,
+                                 const int* __restrict__ slot, int num_segs, int* __restrict__ last_tok,
+                                 int num_slots) {
+  const int sg = blockIdx.x * blockDim.x + threadIdx.x;
+  if (sg >= num_segs) return;
+  const int sl = slot[sg];
+  const int a = start[sg], b = start[sg + 1];
+  if (sl < 0 || sl >= num_slots || b <= a) return;
+  last_tok[sl] = ids[b - 1];
+}
+
+// residual (fp32, in place): x += mult * (y1 + y2);  out = rms_norm(x) * next_w (TO).
+// y1 / y2 are fp32 or bf16 each and optional, as is out.
+template <typename TO, int NT>
+__global__ void add_scaled_rms_norm_kernel(float* __restrict__ x, const void* __restrict__ y1, int y1_bf16,
+                                           long y1_stride, const void* __restrict__ y2, int y2_bf16,
+                                           long y2_stride, float mult, const float* __restrict__ next_w,
+                                           TO* __restrict__ out, int width, float eps) {
+  __shared__ float red[NT / 64];
+  const long row = blockIdx.x;
+  float* xr = x + row * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) {
+    float v = xr[i];
+    if (y1 != nullptr) {
+      float y = ldx(y1, y1_bf16, row * y1_stride + i);
+      if (y2 != nullptr) y += ldx(y2, y2_bf16, row * y2_stride + i);
+      v += mult * y;
+      xr[i] = v;
+    }
+    ss += v * v;
+  }
+  if (out == nullptr) return;
+  ss = block_sum<NT>(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)width + eps);
+  // each thread re-reads only what it wrote itself
+  for (int i = threadIdx.x; i < width; i += NT) st(out, row * width + i, xr[i] * r * next_w[i]);
+}
+
+// out (fp32) = scale * (a / rms(a) * wa + b / rms(b) * wb), one workgroup per row
+template <typename T, int NT>
+__global__ void dual_rms_mean_kernel(float* __restrict__ out, const T* __restrict__ a, long a_stride,
+                                     const T* __restrict__ b, long b_stride, const float* __restrict__ wa,
+                                     const float* __restrict__ wb, int width, float eps, float scale) {
+  __shared__ float red[NT / 64];
+  const long row = blockIdx.x;
+  const T* ar = a + row * a_stride;
+  const T* br = b + row * b_stride;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < width; i += NT) {
+    const float u = ld(ar, i), v = ld(br, i);
+    sa += u * u;
+    sb += v * v;
+  }
+  sa = block_sum<NT>(sa, red);
+  sb = block_sum<NT>(sb, red);
+  const float ra = 1.0f / sqrtf(sa / (float)width + eps), rb = 1.0f / sqrtf(sb / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += NT)
+    out[row * width + i] = scale * (ld(ar, i) * ra * wa[i] + ld(br, i) * rb * wb[i]);
+}
+
+// out = o * sigmoid(g), o fp32 dense rows, g rows g_stride apart
+template <typename TG, typename TO>
+__global__ void sigmoid_gate_kernel(TO* __restrict__ out, const float* __restrict__ o, const TG* __restrict__ g,
+                                    long g_stride, long rows, int n) {
+  const long total = rows * n;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / n;
+    const int c = (int)(i % n);
+    st(out, i, o[i] * sigmoidf_(ld(g, r * g_stride + c)));
+  }
+}
+
 // layer norm with weight and bias, ln(u) = (u - mean) / sqrt(var + eps) * w + b with var
 // the mean squared deviation (two passes), around an fp32 residual x:
 //   y given:            x += ln(y);  cast = x
@@ -113,11 +231,11 @@ __global__ void add_rms_norm_kernel(float* __restrict__ x, const TY* __restrict_
     for (int i = threadIdx.x; i < width; i += NT) st(cast, row * width + i, xr[i]);
 }
 
-// one wave per (row, head): out = o / rms(o) * w * sigmoid(gate)
+// one wave per (row, head): out = o / rms(o) * w * sigmoid(gate), or * silu(gate)
 template <typename TG, typename TO>
 __global__ void head_rms_gate_kernel(TO* __restrict__ out, const float* __restrict__ o,
                                      const float* __restrict__ w, const TG* __restrict__ gate,
-                                     long gate_stride, long pairs, int heads, int dv, float eps) {
+                                     long gate_stride, long pairs, int heads, int dv, float eps, int silu) {
   const long pair = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (pair >= pairs) return;
   const int lane = threadIdx.x & 63;
@@ -129,7 +247,8 @@ __global__ void head_rms_gate_kernel(TO* __restrict__ out, const float* __restri
   ss = ft::wave_sum(ss);
   const float r = 1.0f / sqrtf(ss / (float)dv + eps);
   for (int i = lane; i < dv; i += 64) {
-    const float g = sigmoidf_(ld(gate, row * gate_stride + (long)h * dv + i));
+    const float gp = ld(gate, row * gate_stride + (long)h * dv + i);
+    const float g = silu ? gp * sigmoidf_(gp) : sigmoidf_(gp);
     st(out, (row * heads + h) * dv + i, op[i] * r * w[i] * g);
   }
 }
@@ -188,14 +307,16 @@ __device__ __forceinline__ float gelu_tanh_(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-// rows [gate (ff) | up (ff)]: out = gelu_tanh(gate) * up
+// rows [gate (ff) | up (ff)]: out = gelu_tanh(gate) * up, or relu(gate) * up
 template <typename T>
-__global__ void gelu_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, long gu_stride, long rows, int ff) {
+__global__ void gelu_glu_kernel(T* __restrict__ out, const T* __restrict__ gu, long gu_stride, long rows, int ff,
+                                int relu) {
   const long n = rows * ff;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
     const long r = i / ff;
     const int c = (int)(i % ff);
-    st(out, i, gelu_tanh_(ld(gu, r * gu_stride + c)) * ld(gu, r * gu_stride + ff + c));
+    const float g = ld(gu, r * gu_stride + c);
+    st(out, i, (relu ? fmaxf(g, 0.f) : gelu_tanh_(g)) * ld(gu, r * gu_stride + ff + c));
   }
 }
 
@@ -286,16 +407,16 @@ extern "C" int mx_add_rms_norm(float* x, const void* y, int y_bf16, long y_strid
 
 extern "C" int mx_head_rms_gate(void* out, int out_bf16, const float* o, const float* w,
                                 const void* gate, int gate_bf16, long gate_stride, long rows, int heads,
-                                int dv, float eps, hipStream_t s) {
+                                int dv, float eps, int silu, hipStream_t s) {
   const long pairs = rows * heads;
   if (pairs <= 0) return 0;
   const dim3 grid((unsigned)((pairs + 3) / 4)), block(256);
   if (gate_bf16 && out_bf16)
     hipLaunchKernelGGL((head_rms_gate_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out, o, w,
-                       (const bf16_t*)gate, gate_stride, pairs, heads, dv, eps);
+                       (const bf16_t*)gate, gate_stride, pairs, heads, dv, eps, silu);
   else if (!gate_bf16 && !out_bf16)
     hipLaunchKernelGGL((head_rms_gate_kernel<float, float>), grid, block, 0, s, (float*)out, o, w,
-                       (const float*)gate, gate_stride, pairs, heads, dv, eps);
+                       (const float*)gate, gate_stride, pairs, heads, dv, eps, silu);
   else
     return -1;
   return (int)hipGetLastError();
@@ -343,10 +464,11 @@ extern "C" int mx_clamp_swiglu(void* out, const void* gu, int bf16, long gu_stri
   return (int)hipGetLastError();
 }
 
-extern "C" int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, hipStream_t s) {
+extern "C" int mx_gelu_glu(void* out, const void* gu, int bf16, long gu_stride, long rows, int ff, int relu,
+                           hipStream_t s) {
   if (rows * ff <= 0) return 0;
   MX_DISPATCH_T(bf16, hipLaunchKernelGGL((gelu_glu_kernel<T>), dim3(ew_grid(rows * ff)), dim3(256), 0, s, (T*)out,
-                                         (const T*)gu, gu_stride, rows, ff));
+                                         (const T*)gu, gu_stride, rows, ff, relu));
   return (int)hipGetLastError();
 }
 
@@ -375,5 +497,57 @@ extern "C" int mx_scale_add_rows(float* out, const void* y, int y_bf16, const in
   else
     hipLaunchKernelGGL((scale_add_rows_kernel<float, float>), grid, block, 0, s, out, (const float*)y,
                        rows, (const float*)weights, sigmoid, width, out_rows);
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_pair_embed_add(float* x, const int* ids, const void* table, int bf16, int rows, int width,
+                                 long mul_prev, long mul_cur, int buckets, const int* start, const int* pos0,
+                                 const int* slot, int num_segs, int* last_tok, int num_slots, const void* embed,
+                                 int vocab, float scale, hipStream_t s) {
+  if (rows <= 0 || num_segs <= 0) return 0;
+  if (buckets < 1 || width < 1) return -1;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((pair_embed_add_kernel<T>), dim3(rows), dim3(256), 0, s, x, ids,
+                                         (const T*)table, width, mul_prev, mul_cur, buckets, start, pos0, slot,
+                                         num_segs, last_tok, num_slots, (const T*)embed, vocab, scale));
+  hipLaunchKernelGGL(pair_last_kernel, dim3((num_segs + 63) / 64), dim3(64), 0, s, ids, start, slot, num_segs, last_tok,
+                     num_slots);
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_add_scaled_rms_norm(float* x, const void* y1, int y1_bf16, long y1_stride, const void* y2,
+                                      int y2_bf16, long y2_stride, float mult, const float* next_w, void* out,
+                                      int out_bf16, int rows, int width, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (y1 == nullptr && (y2 != nullptr || out == nullptr)) return -1;
+  if (out_bf16)
+    hipLaunchKernelGGL((add_scaled_rms_norm_kernel<bf16_t, 256>), dim3(rows), dim3(256), 0, s, x, y1, y1_bf16,
+                       y1_stride, y2, y2_bf16, y2_stride, mult, next_w, (bf16_t*)out, width, eps);
+  else
+    hipLaunchKernelGGL((add_scaled_rms_norm_kernel<float, 256>), dim3(rows), dim3(256), 0, s, x, y1, y1_bf16,
+                       y1_stride, y2, y2_bf16, y2_stride, mult, next_w, (float*)out, width, eps);
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_dual_rms_mean(float* out, const void* a, long a_stride, const void* b, long b_stride, int bf16,
+                                const float* wa, const float* wb, int rows, int width, float eps, float scale,
+                                hipStream_t s) {
+  if (rows <= 0) return 0;
+  MX_DISPATCH_T(bf16, hipLaunchKernelGGL((dual_rms_mean_kernel<T, 256>), dim3(rows), dim3(256), 0, s, out,
+                                         (const T*)a, a_stride, (const T*)b, b_stride, wa, wb, width, eps, scale));
+  return (int)hipGetLastError();
+}
+
+extern "C" int mx_sigmoid_gate(void* out, int out_bf16, const float* o, const void* g, int g_bf16, long g_stride,
+                               long rows, int n, hipStream_t s) {
+  if (rows * n <= 0) return 0;
+  const dim3 grid(ew_grid(rows * n)), block(256);
+  if (g_bf16 && out_bf16)
+    hipLaunchKernelGGL((sigmoid_gate_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out, o, (const bf16_t*)g,
+                       g_stride, rows, n);
+  else if (!g_bf16 && !out_bf16)
+    hipLaunchKernelGGL((sigmoid_gate_kernel<float, float>), grid, block, 0, s, (float*)out, o, (const float*)g,
+                       g_stride, rows, n);
+  else
+    return -1;
   return (int)hipGetLastError();
 }

@@ -4,9 +4,12 @@
 //
 // Query head a = h * maps + m (head h, map m) reads key head (h / rep) * maps + m and
 // value head h / rep, rep = heads / kv_heads.  Position i sees key j iff 0 <= i - j
-// (< window when window > 0).  s = q.k * scale, capped to softcap tanh(s / softcap) when
-// softcap > 0; score = s - r1[a] ln(1 + r2[a] (i - j)); weight = softmax over the visible
-// keys, or sigmoid(score + pb[a]) unnormalised.  A softmax may carry a sink: one more
+// (< window when window > 0); with `blocks` the window is a block of the sequence instead
+// (j <= i and i / window == j / window, blocks counted from position 0); with
+// keep_first = f > 0 the positions j < f stay visible whatever the window.
+// s = q.k * scale, capped to softcap tanh(s / softcap) when softcap > 0;
+// score = s - r1[a] ln(1 + r2[a] (i - j)) + dist_bias[min(i - j, nd - 1)][a]; weight =
+// softmax over the visible keys, or sigmoid(score + pb[a]) unnormalised.  A softmax may carry a sink: one more
 // term exp(sink) in its denominator, a key that is always visible and has no value.
 // Queries, scores, weights and sums are fp32; the caches hold fp32 or bf16 rows.
 //
@@ -235,7 +238,7 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
                    int heads, int maps, int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
                    const float* __restrict__ r1, const float* __restrict__ r2, const float* __restrict__ pb,
                    int block_size, int num_blocks, int skip_from, int vec, int lpk, float softcap, int has_sink,
-                   float sink) {
+                   float sink, int blocks, int keep_first, const float* __restrict__ dist_bias, int nd) {
   extern __shared__ float smem[];
   const int row = blockIdx.x, a = blockIdx.y;
   const int hq = heads * maps;
@@ -260,8 +263,10 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
   const long nk = (long)kv_heads * maps * dk, nv = (long)kv_heads * dv;
   const int i = pos0[s] + (row - r0);
   const int last = min(i, kv_len[s] - 1);    // padding rows (empty context) see nothing
-  const int first = window > 0 ? max(0, i - window + 1) : 0;
-  const int nkeys = last - first + 1;
+  const int first = window > 0 ? (blocks ? (i / window) * window : max(0, i - window + 1)) : 0;
+  // kept first positions that lie before the window: keys 0 .. ext-1 go in front of the band
+  const int ext = window > 0 ? max(0, min(min(keep_first, first), last + 1)) : 0;
+  const int nkeys = ext + max(0, last - first + 1);
   const float c1 = r1 != nullptr ? r1[a] : 0.f, c2 = r1 != nullptr ? r2[a] : 0.f;
   const float bias = (sigmoid && pb != nullptr) ? pb[a] : 0.f;
   const int* table = bt + (long)s * bt_stride;
@@ -277,7 +282,8 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
   float mx_ = -INFINITY, l_ = 0.f;
   for (int c0 = wave * 64; c0 < nkeys; c0 += 64 * kWaves) {
     const int cnt = min(64, nkeys - c0);
-    const int j = first + c0 + lane;
+    const int cc = c0 + lane;
+    const int j = cc < ext ? cc : first + cc - ext;
     int slot = -1;
     float z = -INFINITY;
     if (lane < cnt) {
@@ -287,6 +293,7 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
         z = dot_row<TC>(k_cache + (long)slot * nk + (long)kh * dk, q_s, dk, vec != 0) * scale;
         if (softcap > 0.f) z = softcap * tanhf(z / softcap);
         if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)(i - j));
+        if (dist_bias != nullptr) z += dist_bias[(long)min(i - j, nd - 1) * hq + a];
       }
     }
     float p;
@@ -378,12 +385,17 @@ window_attn_kernel(float* __restrict__ out, const float* __restrict__ q, const T
 // ---------------------------------------------------------------------------------
 // scores -> weights in place for the banded products.  S [gk = (g, m)] [(r, t)] [keys]:
 // the rep query heads of a key head stacked along the rows.  grid (rep * rows, gk).
+// The first `ext` columns are the positions 0 .. ext-1 (kept first tokens that lie before
+// the band), column c >= ext is position key0 + c - ext.  A row's visible columns are
+// the kept ones [0, ka) and its window (or block) [c_lo, c_hi].
 // ---------------------------------------------------------------------------------
 template <int NT>
 __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, int first_pos, int key0,
                                     int heads, int maps, int kv_heads, int window, float scale, int sigmoid,
                                     const float* __restrict__ r1, const float* __restrict__ r2,
-                                    const float* __restrict__ pb, float softcap, int has_sink, float sink) {
+                                    const float* __restrict__ pb, float softcap, int has_sink, float sink,
+                                    int blocks, int keep_first, int ext, const float* __restrict__ dist_bias,
+                                    int nd) {
   __shared__ float red[NT / 64];
   const int rep = heads / kv_heads;
   const int rr = blockIdx.x, gk = blockIdx.y;
@@ -392,25 +404,35 @@ __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, i
   const int a = (g * rep + r) * maps + m;
   const int i = first_pos + t;
   float* sp = S + ((long)gk * rep * rows + rr) * keys;
-  // visible columns [c_lo, c_hi]
-  const int c_hi = min(keys - 1, i - key0);
-  const int c_lo = window > 0 ? max(0, i - window + 1 - key0) : 0;
+  // visible columns [0, ka) and [c_lo, c_hi]
+  const int hq = heads * maps;
+  const int first_i = window > 0 ? (blocks ? (i / window) * window : max(0, i - window + 1)) : 0;
+  const int c_hi = min(keys - 1, i - key0 + ext);
+  const int c_lo = max(ext, first_i - key0 + ext);
+  const int ka = window > 0 ? min(c_lo, ext + max(0, keep_first - key0)) : 0;
+  const int nvis = ka + max(0, c_hi - c_lo + 1);
   const float c1 = r1 != nullptr ? r1[a] : 0.f, c2 = r1 != nullptr ? r2[a] : 0.f;
   auto score = [&](int c) {
+    const int d = i - (c < ext ? c : key0 + c - ext);
     float z = sp[c] * scale;
     if (softcap > 0.f) z = softcap * tanhf(z / softcap);
-    if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)(i - key0 - c));
+    if (r1 != nullptr) z -= c1 * logf(1.0f + c2 * (float)d);
+    if (dist_bias != nullptr) z += dist_bias[(long)min(d, nd - 1) * hq + a];
     return z;
   };
-  for (int c = threadIdx.x; c < c_lo; c += NT) sp[c] = 0.f;
-  for (int c = c_hi + 1 + threadIdx.x; c < keys; c += NT) sp[c] = 0.f;
+  for (int c = ka + threadIdx.x; c < min(c_lo, keys); c += NT) sp[c] = 0.f;
+  for (int c = max(c_hi + 1, ka) + threadIdx.x; c < keys; c += NT) sp[c] = 0.f;
   if (sigmoid) {
     const float bias = pb != nullptr ? pb[a] : 0.f;
-    for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) sp[c] = sigmoidf_(score(c) + bias);
+    for (int u = threadIdx.x; u < nvis; u += NT) {
+      const int c = u < ka ? u : c_lo + u - ka;
+      sp[c] = sigmoidf_(score(c) + bias);
+    }
     return;
   }
   float mx_ = -INFINITY;
-  for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) {
+  for (int u = threadIdx.x; u < nvis; u += NT) {
+    const int c = u < ka ? u : c_lo + u - ka;
     const float z = score(c);
     sp[c] = z;                         // each thread re-reads only its own columns
     mx_ = fmaxf(mx_, z);
@@ -423,7 +445,8 @@ __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, i
   for (int w = 0; w < NT / 64; ++w) mx_ = fmaxf(mx_, red[w]);
   if (has_sink) mx_ = fmaxf(mx_, sink);
   float sum = 0.f;
-  for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) {
+  for (int u = threadIdx.x; u < nvis; u += NT) {
+    const int c = u < ka ? u : c_lo + u - ka;
     const float p = expf(sp[c] - mx_);
     sp[c] = p;
     sum += p;
@@ -431,7 +454,10 @@ __global__ void band_weights_kernel(float* __restrict__ S, int rows, int keys, i
   sum = block_sum<NT>(sum, red);
   if (has_sink) sum += expf(sink - mx_);
   const float inv = sum > 0.f ? 1.0f / sum : 0.f;
-  for (int c = c_lo + threadIdx.x; c <= c_hi; c += NT) sp[c] *= inv;
+  for (int u = threadIdx.x; u < nvis; u += NT) {
+    const int c = u < ka ? u : c_lo + u - ka;
+    sp[c] *= inv;
+  }
 }
 
 // one wave per (row, head): o = a1 - lam a2; o / rms(o) * post * sigmoid(gate)
@@ -517,9 +543,10 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
                                    int kv_heads, int dk, int dv, int window, float scale, int sigmoid,
                                    const float* r1, const float* r2, const float* pb, int block_size,
                                    int num_blocks, int skip_from, float softcap, int has_sink, float sink,
-                                   hipStream_t s) {
+                                   int blocks, int keep_first, const float* dist_bias, int nd, hipStream_t s) {
   if (num_segs <= 0 || total_rows <= 0) return 0;
   if (dv < 1 || dv > mx_window_max_dv() || dk < 1 || heads % kv_heads || maps < 1) return -1;
+  if (keep_first < 0 || (dist_bias != nullptr && nd < 1) || (blocks && window < 1)) return -1;
   const int hq = heads * maps;
   if (total_rows > 0x7fffffffL || hq > 65535) return -2;
   const long es = cache_bf16 ? 2 : 4;
@@ -539,7 +566,7 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
                                                (const T*)k_cache, (const T*)v_cache, start, pos0, kv_len, bt,  \
                                                bt_stride, num_segs, heads, maps, kv_heads, dk, dv, window, scale, \
                                                sigmoid, r1, r2, pb, block_size, num_blocks, skip_from, vec, lpk,  \
-                                               softcap, has_sink, sink))
+                                               softcap, has_sink, sink, blocks, keep_first, dist_bias, nd))
   if (vecv) MX_WATTN(true);
   else MX_WATTN(false);
 #undef MX_WATTN
@@ -549,12 +576,16 @@ extern "C" int mx_window_attention(float* out, const float* q, const void* k_cac
 extern "C" int mx_band_weights(float* S, int gk, int rep_rows_total, int rows, int keys, int first_pos, int key0,
                                int heads, int maps, int kv_heads, int window, float scale, int sigmoid,
                                const float* r1, const float* r2, const float* pb, float softcap, int has_sink,
-                               float sink, hipStream_t s) {
+                               float sink, int blocks, int keep_first, int ext, const float* dist_bias, int nd,
+                               hipStream_t s) {
   if (gk <= 0 || rep_rows_total <= 0 || keys <= 0) return 0;
   if (heads % kv_heads || gk != kv_heads * maps || rep_rows_total != heads / kv_heads * rows || gk > 65535) return -1;
+  if (keep_first < 0 || ext < 0 || ext > keys || ext > key0 || (dist_bias != nullptr && nd < 1) ||
+      (blocks && window < 1))
+    return -1;
   hipLaunchKernelGGL((band_weights_kernel<256>), dim3((unsigned)rep_rows_total, (unsigned)gk), dim3(256), 0, s, S,
                      rows, keys, first_pos, key0, heads, maps, kv_heads, window, scale, sigmoid, r1, r2, pb, softcap,
-                     has_sink, sink);
+                     has_sink, sink, blocks, keep_first, ext, dist_bias, nd);
   return (int)hipGetLastError();
 }
 
