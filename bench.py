@@ -181,7 +181,7 @@ def main():
     ap.add_argument("--engine-compare", default="", metavar="MODELS",
                     help="instead of the headline benchmark: engine-level prefill / decode throughput "
                          "of these registry models side by side (comma separated, random weights), "
-                         "e.g. kerarax-2k,nulazen-2k,bagasun-2k,llama-2k-4l (bench/engine_compare.py)")
+                         "e.g. fufipel-2k,kerarax-2k,nulazen-2k,bagasun-2k,llama-2k-4l (bench/engine_compare.py)")
     ap.add_argument("--compare-prompts", default="512,2048,4096")
     ap.add_argument("--compare-batches", default="1,8,32")
     ap.add_argument("--compare-dtype", default="bfloat16", choices=["bfloat16", "float32"])
